@@ -1,0 +1,201 @@
+#!/usr/bin/env python3
+"""Benchmark of the int4 dequant-matmul path on one MI355X.
+
+Headline (BASELINE.json metric, configs[1]): int4 affine group-64 decode GEMV
+at 8B shapes, M=1: (K=4096,N=14336), (K=14336,N=4096), (K=4096,N=6144).
+One step = the three GEMVs on one weight set; steps rotate over distinct
+weight sets whose total exceeds the 256 MB last-level cache, so every step
+streams its weights from HBM. Inputs are resident in HBM before timing.
+
+Prints ONE JSON line: value = algorithmic weight GB/s over the timed steps,
+plus `roofline` (HBM) and `cpu_baseline` (the CPU oracle on the host cores).
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense f16 MFMA, published
+
+GEMV_SHAPES = [("ffn_gate_or_up", 4096, 14336), ("ffn_down", 14336, 4096), ("qkv_fused", 4096, 6144)]
+
+
+def make_desc(capi, bits, K, N, M, bufs, kernel=0):
+    return capi.MatmulDesc(bits=bits, affine=1, out_f32=0, kernel=kernel, M=M, N=N, k_packed=K * bits // 32,
+                           scales_per_row=K // 64, out=bufs["out"], in_=bufs["in"], scales=bufs["s"],
+                           weights=bufs["w"], biases=bufs["b"])
+
+
+def upload_set(ctx, synth, K, N, bits, salt, M=1):
+    w = synth.packed_weights(N, K, bits=bits, salt=salt)
+    s = synth.scales(N, K, salt=salt)
+    b = synth.biases(N, K, s, "A", salt=salt)
+    x = synth.activations(M, K, salt=salt)
+    bufs = {}
+    for key, arr in (("w", w), ("s", s), ("b", b), ("in", x)):
+        bufs[key] = ctx.alloc(arr.nbytes)
+        ctx.upload(bufs[key], arr)
+    bufs["out"] = ctx.alloc(M * N * 2)
+    return bufs, (x, w, s, b)
+
+
+def timed_graph(ctx, launches, reps=1):
+    """Record `launches` (callables) into one command buffer, replay once untimed, then time `reps` replays."""
+    ctx.record_begin()
+    for fn in launches:
+        fn()
+    cb = ctx.record_end()
+    ctx.submit(cb)
+    ctx.sync()
+    e0, e1 = ctx.event(), ctx.event()
+    ctx.event_record(e0)
+    for _ in range(reps):
+        ctx.submit(cb)
+    ctx.event_record(e1)
+    ms = ctx.elapsed_ms(e0, e1)
+    ctx.event_destroy(e0)
+    ctx.event_destroy(e1)
+    ctx.cmdbuf_destroy(cb)
+    return ms / reps
+
+
+def verify(ctx, oracle, capi, desc, host, bits, K, N, M, f16w=False):
+    """Validate before timing: a launch that did not run times as ~0 and must never be reported."""
+    x, w, s, b = host
+    ctx.fill(desc.out, 0xFF, M * N * 2)
+    ctx.matmul(desc)
+    y = ctx.download(desc.out, M * N * 2, np.float16).astype(np.float64).reshape(M, N)
+    rows = min(M, 4)
+    mode = oracle.MODE_F16W if f16w else oracle.MODE_FORMULA_F32
+    ref = oracle.gemm(mode, bits, True, rows, N, K, x[:rows], w, s, b, threads=oracle.max_threads())
+    err = float(np.max(np.abs(y[:rows] - ref) / (np.abs(ref) + 1e-2)))
+    if not np.all(np.isfinite(y)) or err >= 1e-2:
+        raise SystemExit("bench: output check failed (K=%d N=%d M=%d): rel err %.3e" % (K, N, M, err))
+    return err
+
+
+def cpu_baseline(oracle, synth, budget_s=12.0):
+    """The CPU oracle (a port of the reference's JS kernel-test reference) on this host's cores."""
+    threads = oracle.max_threads()
+    sets = []
+    for _, K, N in GEMV_SHAPES:
+        w = synth.packed_weights(N, K, salt=99)
+        s = synth.scales(N, K, salt=99)
+        sets.append((K, N, synth.activations(1, K, salt=99), w, s, synth.biases(N, K, s, "A", salt=99)))
+    nbytes = sum(synth.weight_bytes(N, K) for _, K, N in GEMV_SHAPES)
+
+    def one_pass(th):
+        t0 = time.perf_counter()
+        for K, N, x, w, s, b in sets:
+            oracle.gemm(oracle.MODE_JS, 4, True, 1, N, K, x, w, s, b, threads=th)
+        return time.perf_counter() - t0
+
+    one_pass(threads)
+    t_multi, t_end = [], time.perf_counter() + budget_s * 0.5
+    while time.perf_counter() < t_end or len(t_multi) < 3:
+        t_multi.append(one_pass(threads))
+    t_single, t_end = [], time.perf_counter() + budget_s * 0.5
+    while time.perf_counter() < t_end or len(t_single) < 2:
+        t_single.append(one_pass(1))
+    med_m, med_s = float(np.median(t_multi)), float(np.median(t_single))
+    return {
+        "value": round(nbytes / med_m / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+        "sample": "%d passes of the three configs[1] GEMVs (80.2 MB of weights each) on %d OpenMP threads; "
+                  "single thread: %.3f GB/s over %d passes" % (len(t_multi), threads, nbytes / med_s / 1e9, len(t_single)),
+        "single_thread_value": round(nbytes / med_s / 1e9, 3),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=240)
+    ap.add_argument("--warmup", type=int, default=24)
+    ap.add_argument("--sets", type=int, default=8, help="distinct weight sets rotated through (8 x 80 MB > 256 MB cache)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the per-shape, GEMM, MoE and int3 extras")
+    ap.add_argument("--option", action="append", default=[], help="name=value launch knob (ztvm_set_option)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py: this path is built and measured on ONE GPU; --gpus %d is not supported "
+                         "(sharding is design-only, see DESIGN.md)" % args.gpus)
+
+    pkg = importlib.import_module("zero-tvm_amd")
+    capi = pkg.capi
+    synth = importlib.import_module("zero-tvm_amd.host.synth")
+    from oracle import oracle
+
+    ctx = capi.Context(0)
+    for opt in args.option:
+        k, v = opt.split("=")
+        ctx.set_option(k, int(v))
+    info = ctx.device_info()
+
+    # ---- headline: rotating weight sets, three GEMVs per step ------------------
+    sets = []
+    for r in range(args.sets):
+        per_shape = []
+        for i, (_, K, N) in enumerate(GEMV_SHAPES):
+            bufs, host = upload_set(ctx, synth, K, N, 4, salt=10 * r + i)
+            desc = make_desc(capi, 4, K, N, 1, bufs)
+            if r == 0:
+                verify(ctx, oracle, capi, desc, host, 4, K, N, 1)
+            per_shape.append(desc)
+        sets.append(per_shape)
+    step_bytes = sum(synth.weight_bytes(N, K) for _, K, N in GEMV_SHAPES)
+
+    def step(i):
+        for desc in sets[i % args.sets]:
+            ctx.matmul(desc)
+
+    for i in range(args.warmup):
+        step(i)
+    ctx.sync()
+    ms_total = timed_graph(ctx, [lambda i=i: step(i) for i in range(args.steps)])
+    ms_per_step = ms_total / args.steps
+    gbs = step_bytes / (ms_per_step * 1e-3) / 1e9
+    launches = 3 * args.steps
+    avg_launch_us = ms_total * 1e3 / launches
+
+    result = {
+        "metric": "int4 GEMV GB/s (% of HBM peak) at M=1; prefill GEMM TFLOP/s at M=512",
+        "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int4 weights (u32-packed), f16 activations, f32 accumulate", "data": "synthetic",
+        "config": {"workload": "configs[1]: int4 affine g64 decode GEMV, M=1, (4096->14336)+(14336->4096)+(4096->6144) "
+                               "per step, %d rotating weight sets" % args.sets,
+                   "device": info["name"], "compute_units": info["compute_units"]},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "ztvm::gemv_kernel<4,true,64,*>", "bytes_per_launch": step_bytes / 3.0,
+                     "avg_launch_us": round(avg_launch_us, 3), "launches": launches},
+    }
+
+    if not args.no_extra:
+        extra = {}
+        # per shape, each alone over its rotating sets
+        for i, (name, K, N) in enumerate(GEMV_SHAPES):
+            reps = 40
+            ms = timed_graph(ctx, [lambda d=sets[j % args.sets][i]: ctx.matmul(d) for j in range(reps * args.sets)]) / (reps * args.sets)
+            wb = synth.weight_bytes(N, K)
+            extra["gemv_%s_K%d_N%d" % (name, K, N)] = {"us": round(ms * 1e3, 3), "GB/s": round(wb / ms / 1e6, 1),
+                                                       "hbm_frac": round(wb / ms / 1e6 / HBM_PEAK_GBS, 4)}
+        result["extra"] = extra
+
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(oracle, synth)
+
+    ctx.close()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

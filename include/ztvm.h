@@ -1,0 +1,190 @@
+/*
+ * libztvm_hip — C ABI of the MI355X (gfx950) int4/int3 group-quantized
+ * dequant-matmul path: M=1 decode GEMV, small-M GEMV, prefill GEMM and the
+ * MoE gathered GEMV.
+ *
+ * The boundary it replaces is the WebGPU dispatch surface of the reference
+ * engine (paths relative to the reference's root):
+ *   uniformBuf()  src/zero-tvm/engine-core.ts:53-65     PODArgs uniform
+ *   bg()          src/zero-tvm/engine-core.ts:76-92     bind group, binding i = array index i
+ *   dispatch()    src/zero-tvm/engine-core.ts:2151-2179 one compute pass
+ * and the binding contract of the kernel generator
+ *   src/compiler/shaders/int4_matmul.gen.ts:24-30, :211-226
+ *   (0 out / 1 in / 2 scales / 3 weights / 4 PODArgs / 5 biases / 6 ids).
+ *
+ * Conventions: every entry point is extern "C", takes plain pointers and
+ * sizes, returns 0 on success or a negative ZTVM_E_* code, never throws and
+ * never falls back to a CPU path. Device memory is named by its 64-bit device
+ * address. All work is enqueued on the context's single HIP stream in call
+ * order (the reference's queue order); only ztvm_download, ztvm_sync and
+ * ztvm_event_elapsed_ms block. The caller owns every buffer.
+ */
+#ifndef ZTVM_H
+#define ZTVM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ZTVM_ABI_VERSION 1
+
+#if defined(__GNUC__)
+#define ZTVM_API __attribute__((visibility("default")))
+#else
+#define ZTVM_API
+#endif
+
+enum {
+  ZTVM_OK = 0,
+  ZTVM_E_INVALID = -1,     /* descriptor or argument rejected before any GPU work */
+  ZTVM_E_HIP = -2,         /* a HIP runtime call failed; see ztvm_last_error */
+  ZTVM_E_UNSUPPORTED = -3, /* an explicitly requested kernel cannot run this descriptor */
+  ZTVM_E_NODEVICE = -4     /* no gfx950 device visible */
+};
+
+/* Kernel families. AUTO picks by M; naming a family that cannot run the
+ * descriptor is an error, never a silent substitution (the rule of
+ * pickChunkGemm, src/zero-tvm/engine-core.ts:220-245). */
+enum {
+  ZTVM_KERNEL_AUTO = 0,
+  ZTVM_KERNEL_GEMV = 1,   /* one pass per activation row; replaces int4_matmul[_sg|_tiled|_vec4|_vec4h][_affine][_q3][_moe] */
+  ZTVM_KERNEL_SKINNY = 2, /* 2 <= M <= 64, weights read once; replaces int4_matmul_batched_m4 / _batched_dyn[_affine] */
+  ZTVM_KERNEL_GEMM = 3    /* MFMA tile GEMM; replaces int4_matmul_tiled_st / _sg_e1 / _sg_e5 [_affine] */
+};
+
+typedef struct ztvm_ctx ztvm_ctx;
+typedef struct ztvm_cmdbuf ztvm_cmdbuf;
+typedef struct ztvm_event ztvm_event;
+
+/* One quantized matmul dispatch: the PODArgs uniform
+ * (src/compiler/shaders/int4_matmul.gen.ts:216-225, :645-650) plus the bind
+ * group entries, with the variant options of Int4MatmulOpts (:32-134) that
+ * change arithmetic (bits, affine, outF32, moe). Options that only chose a
+ * WGSL tiling (rowsPerWG, subgroups, vec4, vec4Half, the grid) have no
+ * counterpart: N, M, tokens and slots define the work.
+ *
+ *   Y[m,n] = sum_k A[m,k] * w[n,k],  f32 accumulation, f16 (or f32) store
+ *   affine=1: w = q*s + b, group 64     affine=0: w = (q-7)*s, group 32
+ *   bits=4: k_packed = K/8, value k at (W[n,k>>3] >> 4*(k&7)) & 15
+ *   bits=3: k_packed = 3K/32, row is an LSB-first bitstream, value k at bits [3k,3k+3)
+ *
+ * Dense (slots == 0): A is [M,K] f16 row-major, Y is [M,N]; rows >= M are
+ * neither read nor written. MoE (slots > 0, M must be 1): for every
+ * (token < tokens, slot < slots) expert = ids[token*ids_stride + slot],
+ * weights/scales/biases are [experts][N][...] stacks, the input row starts at
+ * element token*in_tok_stride + slot*in_slot_stride of `in` and the output
+ * row at token*out_tok_stride + slot*out_slot_stride of `out`
+ * (:236-253). A pair whose expert id is >= experts (when experts != 0) is
+ * skipped, so a bad id cannot fault the GPU. */
+typedef struct ztvm_matmul_desc {
+  uint32_t bits;           /* 4 | 3 */
+  uint32_t affine;         /* 0 | 1 */
+  uint32_t out_f32;        /* 0: f16 output, 1: f32 output (LM head) */
+  uint32_t kernel;         /* ZTVM_KERNEL_* */
+  uint32_t M;              /* PODArgs.M_ROWS (1 for GEMV dispatches) */
+  uint32_t N;              /* PODArgs.packGridDimX */
+  uint32_t k_packed;       /* PODArgs.K_PACKED, u32 words per weight row */
+  uint32_t scales_per_row; /* PODArgs.SCALES_PER_ROW = K/group */
+  uint32_t slots;          /* 0 = dense; else grid z of the MoE dispatch */
+  uint32_t tokens;         /* grid y of the MoE dispatch (ignored when dense) */
+  uint32_t in_slot_stride; /* PODArgs.IN_SLOT_STRIDE, f16 elements */
+  uint32_t out_slot_stride;
+  uint32_t in_tok_stride;
+  uint32_t out_tok_stride;
+  uint32_t ids_stride;
+  uint32_t experts;        /* stack height for the id guard; 0 = unchecked */
+  uint64_t out;            /* binding 0 (device address incl. region offset) */
+  uint64_t in;             /* binding 1 */
+  uint64_t scales;         /* binding 2 */
+  uint64_t weights;        /* binding 3 */
+  uint64_t biases;         /* binding 5, affine only */
+  uint64_t ids;            /* binding 6, MoE only */
+} ztvm_matmul_desc;
+
+/* ---- context ----------------------------------------------------------- */
+
+/* Replaces requestAdapter/requestDevice (src/lib/index.ts:210-377): binds a
+ * gfx950 device and creates the stream every later call is ordered on. */
+ZTVM_API int ztvm_create(int device, ztvm_ctx** out);
+ZTVM_API void ztvm_destroy(ztvm_ctx* ctx);
+
+/* Text of the last failure on this context (or of the last context-less
+ * failure when ctx is NULL). Replaces pushErrorScope/uncapturederror
+ * (tests/kernels/gpu.mjs:59-62). Never NULL. */
+ZTVM_API const char* ztvm_last_error(ztvm_ctx* ctx);
+
+ZTVM_API int ztvm_abi_version(void);
+
+/* Device facts the host layer reports: name, compute units, bytes of HBM. */
+ZTVM_API int ztvm_device_info(ztvm_ctx* ctx, char* name, size_t name_len, uint32_t* compute_units, uint64_t* hbm_bytes);
+
+/* ---- buffers (device.createBuffer / queue.writeBuffer / mapAsync) ------- */
+
+/* createBuffer (src/zero-tvm/engine-core.ts:36-41). Address is 256-byte aligned. */
+ZTVM_API int ztvm_alloc(ztvm_ctx* ctx, size_t bytes, uint64_t* dptr);
+ZTVM_API int ztvm_free(ztvm_ctx* ctx, uint64_t dptr);
+/* queue.writeBuffer (src/zero-tvm/engine-core.ts:61-63): the source may be reused on return. */
+ZTVM_API int ztvm_upload(ztvm_ctx* ctx, uint64_t dst, size_t dst_off, const void* src, size_t bytes);
+/* copyBufferToBuffer + mapAsync (tests/kernels/gpu.mjs:95-121): blocks until earlier work finished. */
+ZTVM_API int ztvm_download(ztvm_ctx* ctx, void* dst, uint64_t src, size_t src_off, size_t bytes);
+/* Fill with a repeated byte, ordered on the stream (a kernel, so it may be recorded). */
+ZTVM_API int ztvm_fill(ztvm_ctx* ctx, uint64_t dst, size_t dst_off, int byte, size_t bytes);
+ZTVM_API int ztvm_sync(ztvm_ctx* ctx);
+
+/* ---- dispatch ----------------------------------------------------------- */
+
+/* Pure CPU check of a descriptor against the generator's own legality rules
+ * (src/compiler/shaders/int4_matmul.gen.ts:172-197) and the layout contract;
+ * needs no GPU. `why` receives the reason on failure. */
+ZTVM_API int ztvm_matmul_validate(const ztvm_matmul_desc* desc, char* why, size_t why_len);
+
+/* Which family AUTO resolves to for this descriptor (ZTVM_KERNEL_*), or a
+ * negative error. Pure CPU. Replaces resolveMatmul / pickChunkGemm
+ * (src/zero-tvm/variants.ts:239-388, src/zero-tvm/engine-core.ts:220-245). */
+ZTVM_API int ztvm_matmul_resolve(const ztvm_matmul_desc* desc);
+
+/* bg() + dispatch() of one matmul (src/zero-tvm/engine-core.ts:76-92,
+ * :2151-2179; call sites :2290, :2312, :2343-2347, :2517-2524, :2543-2549,
+ * :4280-4293, :4386-4390). Validates, then enqueues. */
+ZTVM_API int ztvm_matmul(ztvm_ctx* ctx, const ztvm_matmul_desc* desc);
+
+/* Dequantize a weight stack to [N,K] f16 (out_f32=0) or f32 (out_f32=1):
+ * w = fl32(q*s + b) (or (q-7)*s), f16 = RNE of that. Uses bits, affine, N,
+ * k_packed, scales_per_row, weights, scales, biases and out of `desc`.
+ * Replaces the CPU dequantAffineSplit of src/zero-tvm/mlx-weights.ts:598-667
+ * and is the bit-exact parity target. */
+ZTVM_API int ztvm_dequant(ztvm_ctx* ctx, const ztvm_matmul_desc* desc);
+
+/* ---- command buffers (createCommandEncoder / finish / queue.submit) ------ */
+
+/* Between begin and end, ztvm_matmul / ztvm_dequant / ztvm_fill calls are
+ * recorded instead of run (src/zero-tvm/engine-core.ts:2565-2570 records a
+ * whole token into one encoder). Uploads, downloads and syncs are rejected
+ * while recording. */
+ZTVM_API int ztvm_record_begin(ztvm_ctx* ctx);
+ZTVM_API int ztvm_record_end(ztvm_ctx* ctx, ztvm_cmdbuf** out);
+ZTVM_API int ztvm_submit(ztvm_ctx* ctx, ztvm_cmdbuf* cb);
+ZTVM_API void ztvm_cmdbuf_destroy(ztvm_cmdbuf* cb);
+
+/* ---- timing (timestamp-query, src/zero-tvm/engine-core.ts:94-102) -------- */
+
+ZTVM_API int ztvm_event_create(ztvm_ctx* ctx, ztvm_event** out);
+ZTVM_API void ztvm_event_destroy(ztvm_event* ev);
+ZTVM_API int ztvm_event_record(ztvm_ctx* ctx, ztvm_event* ev);
+/* Blocks until `stop` completed; milliseconds between the two records. */
+ZTVM_API int ztvm_event_elapsed_ms(ztvm_ctx* ctx, ztvm_event* start, ztvm_event* stop, float* ms);
+
+/* ---- launch tuning -------------------------------------------------------- */
+
+/* Named integer knobs for measurement sweeps (e.g. "gemv.wg_per_cu"). Unknown
+ * names are ZTVM_E_INVALID. Defaults are the measured best. */
+ZTVM_API int ztvm_set_option(ztvm_ctx* ctx, const char* name, int value);
+ZTVM_API int ztvm_get_option(ztvm_ctx* ctx, const char* name, int* value);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ZTVM_H */

@@ -1,0 +1,147 @@
+"""ctypes wrapper over the CPU oracle (oracle/ztvm_oracle.c).
+
+Test infrastructure only: imported by tests/, the smoke check and the
+bench's cpu_baseline leg. Nothing in the product package imports it.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "_build", "libztvm_oracle.so")
+
+MODE_JS, MODE_FORMULA_F64, MODE_FORMULA_F32, MODE_F16W = 0, 1, 2, 3
+
+
+def build(force=False):
+    """Compile the oracle with gcc (seconds)."""
+    if force or not os.path.exists(_LIB_PATH):
+        subprocess.check_call(["make", "-s", "-B", "-C", _HERE])
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        build()
+        L = C.CDLL(_LIB_PATH)
+        u16p, u32p, f32p, f64p, u8p = (C.POINTER(t) for t in (C.c_uint16, C.c_uint32, C.c_float, C.c_double, C.c_uint8))
+        L.zo_f32_to_f16.restype, L.zo_f32_to_f16.argtypes = C.c_uint16, [C.c_float]
+        L.zo_f16_to_f32.restype, L.zo_f16_to_f32.argtypes = C.c_float, [C.c_uint16]
+        L.zo_f32_to_f16_array.argtypes = [f32p, u16p, C.c_size_t]
+        L.zo_f16_to_f32_array.argtypes = [u16p, f32p, C.c_size_t]
+        L.zo_mulberry32.restype, L.zo_mulberry32.argtypes = C.c_double, [u32p]
+        L.zo_reference_gemv_case.argtypes = [C.c_uint32, C.c_uint32, C.c_uint32, C.c_int, C.c_int, u16p, u16p, u16p, u32p]
+        for f in (L.zo_unpack4, L.zo_unpack3, L.zo_unpack3_window):
+            f.restype, f.argtypes = C.c_uint32, [u32p, C.c_uint32]
+        L.zo_pack3.argtypes = [u8p, C.c_uint32, u32p]
+        L.zo_pack4.argtypes = [u8p, C.c_uint32, u32p]
+        L.zo_dequant_f32.restype = C.c_float
+        L.zo_dequant_f32.argtypes = [C.c_uint32, C.c_uint16, C.c_uint16, C.c_int]
+        L.zo_dequant_f16.restype = C.c_uint16
+        L.zo_dequant_f16.argtypes = [C.c_uint32, C.c_uint16, C.c_uint16, C.c_int]
+        L.zo_dequant_matrix.argtypes = [C.c_uint32, C.c_int, C.c_uint32, C.c_uint32, u32p, u16p, u16p, f32p, u16p]
+        L.zo_gemm.argtypes = [C.c_int, C.c_uint32, C.c_int, C.c_uint32, C.c_uint32, C.c_uint32, u16p, C.c_uint32,
+                              u32p, u16p, u16p, f64p, C.c_int]
+        L.zo_moe_gemv.argtypes = [C.c_int, C.c_uint32] + [C.c_uint32] * 9 + [u32p, u16p, u32p, u16p, u16p, f64p, C.c_int]
+        L.zo_max_threads.restype = C.c_int
+        _lib = L
+    return _lib
+
+
+def _p(a, ct):
+    return None if a is None else a.ctypes.data_as(C.POINTER(ct))
+
+
+def _c(a, dt):
+    return None if a is None else np.ascontiguousarray(a, dtype=dt)
+
+
+def f32_to_f16_bits(x):
+    x = _c(x, np.float32).ravel()
+    out = np.empty(x.size, np.uint16)
+    lib().zo_f32_to_f16_array(_p(x, C.c_float), _p(out, C.c_uint16), x.size)
+    return out
+
+
+def f16_bits_to_f32(h):
+    h = _c(h, np.uint16).ravel()
+    out = np.empty(h.size, np.float32)
+    lib().zo_f16_to_f32_array(_p(h, C.c_uint16), _p(out, C.c_float), h.size)
+    return out
+
+
+def mulberry32(seed, n):
+    st = C.c_uint32(seed & 0xFFFFFFFF)
+    L = lib()
+    return np.array([L.zo_mulberry32(C.byref(st)) for _ in range(n)], np.float64)
+
+
+def reference_gemv_case(N, K, affine, q3, seed=1):
+    """The seeded vector of the reference's own GEMV kernel test."""
+    KP = K * 3 // 32 if q3 else K // 8
+    SPR = K // (64 if affine else 32)
+    x = np.empty(K, np.uint16)
+    s = np.empty(N * SPR, np.uint16)
+    b = np.zeros(N * SPR, np.uint16)
+    w = np.empty(N * KP, np.uint32)
+    lib().zo_reference_gemv_case(seed, N, K, int(affine), int(q3), _p(x, C.c_uint16), _p(s, C.c_uint16),
+                                 _p(b, C.c_uint16), _p(w, C.c_uint32))
+    return x, s.reshape(N, SPR), (b.reshape(N, SPR) if affine else None), w.reshape(N, KP)
+
+
+def unpack(bits, row_words, k, window=False):
+    row = _c(row_words, np.uint32)
+    f = lib().zo_unpack4 if bits == 4 else (lib().zo_unpack3_window if window else lib().zo_unpack3)
+    return f(_p(row, C.c_uint32), k)
+
+
+def pack(bits, values):
+    v = _c(values, np.uint8).ravel()
+    K = v.size
+    out = np.zeros(K * bits // 32, np.uint32)
+    (lib().zo_pack3 if bits == 3 else lib().zo_pack4)(_p(v, C.c_uint8), K, _p(out, C.c_uint32))
+    return out
+
+
+def dequant_scalar(q, s16, b16, affine, f16=False):
+    L = lib()
+    return (L.zo_dequant_f16 if f16 else L.zo_dequant_f32)(int(q), int(s16), int(b16), int(affine))
+
+
+def dequant_matrix(bits, affine, N, K, weights, scales, biases, want="f32"):
+    w, s, b = _c(weights, np.uint32), _c(scales, np.uint16), _c(biases, np.uint16)
+    o32 = np.empty((N, K), np.float32) if want in ("f32", "both") else None
+    o16 = np.empty((N, K), np.uint16) if want in ("f16", "both") else None
+    lib().zo_dequant_matrix(bits, int(affine), N, K, _p(w, C.c_uint32), _p(s, C.c_uint16), _p(b, C.c_uint16),
+                            _p(o32, C.c_float), _p(o16, C.c_uint16))
+    return (o32, o16) if want == "both" else (o32 if o32 is not None else o16)
+
+
+def gemm(mode, bits, affine, M, N, K, A, weights, scales, biases, lda=None, threads=1):
+    """Y[M,N] float64, unrounded. A is f16 bit patterns."""
+    A, w, s, b = _c(A, np.uint16), _c(weights, np.uint32), _c(scales, np.uint16), _c(biases, np.uint16)
+    Y = np.empty((M, N), np.float64)
+    lib().zo_gemm(mode, bits, int(affine), M, N, K, _p(A, C.c_uint16), lda or K, _p(w, C.c_uint32),
+                  _p(s, C.c_uint16), _p(b, C.c_uint16), _p(Y, C.c_double), threads)
+    return Y
+
+
+def moe_gemv(mode, bits, N, K, tokens, slots, strides, ids, x, weights, scales, biases, out_elems, threads=1):
+    """strides = (in_slot, out_slot, in_tok, out_tok, ids_stride); returns float64[out_elems] (zeros where unwritten)."""
+    ids, x = _c(ids, np.uint32), _c(x, np.uint16)
+    w, s, b = _c(weights, np.uint32), _c(scales, np.uint16), _c(biases, np.uint16)
+    out = np.zeros(out_elems, np.float64)
+    lib().zo_moe_gemv(mode, bits, N, K, tokens, slots, *[int(v) for v in strides], _p(ids, C.c_uint32),
+                      _p(x, C.c_uint16), _p(w, C.c_uint32), _p(s, C.c_uint16), _p(b, C.c_uint16),
+                      _p(out, C.c_double), threads)
+    return out
+
+
+def max_threads():
+    return lib().zo_max_threads()

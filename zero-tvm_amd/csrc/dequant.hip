@@ -1,0 +1,126 @@
+// Weight dequantization to a dense [N,K] matrix, plus the byte-fill kernel.
+//
+// The dequantized value is the bit-exact parity target of the whole family:
+//   affine     w = fl32(q*s + b)     (src/zero-tvm/mlx-weights.ts:637-648)
+//   symmetric  w = fl32((q-7)*s)     (src/compiler/shaders/int4_matmul.gen.ts:17-19)
+// q*s is exact in f32 (<= 4 bits x 11 bits), so a single fused multiply-add
+// rounds once, exactly like the reference's f64 expression stored to f32.
+// The f16 form is the RNE of that f32 value (:651-660 of mlx-weights.ts).
+#include "internal.h"
+#include "quant.h"
+
+namespace ztvm {
+namespace {
+
+struct DequantParams {
+  void* out;
+  const _Float16* scales;
+  const uint32_t* weights;
+  const _Float16* biases;
+  uint32_t N, K, k_packed, spr, nchunks;
+  uint32_t out_f32;
+};
+
+struct __attribute__((packed, aligned(4))) Words3 {
+  uint32_t a, b, c;
+};
+
+template <int BITS, bool AFFINE>
+__global__ __launch_bounds__(256) void dequant_kernel(const DequantParams p) {
+  const uint64_t idx = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+  const uint64_t total = (uint64_t)p.N * p.nchunks;
+  if (idx >= total) return;
+  const uint32_t n = (uint32_t)(idx / p.nchunks), c = (uint32_t)(idx % p.nchunks);
+  const uint32_t g = AFFINE ? (c >> 1) : c;
+  const float s = (float)p.scales[(size_t)n * p.spr + g];
+  const float b = AFFINE ? (float)p.biases[(size_t)n * p.spr + g] : 0.f;
+
+  uint32_t q[32];
+  if (BITS == 4) {
+    const u32x4 v = *reinterpret_cast<const u32x4*>(p.weights + (size_t)n * p.k_packed + (size_t)c * 4);
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 32; i++) q[i] = (w[i >> 3] >> (4 * (i & 7))) & 15u;
+  } else {
+    const Words3 v = *reinterpret_cast<const Words3*>(p.weights + (size_t)n * p.k_packed + (size_t)c * 3);
+    const uint64_t lo = (uint64_t)v.a | ((uint64_t)v.b << 32);  // stream bits 0..63
+    const uint64_t hi = (uint64_t)v.b | ((uint64_t)v.c << 32);  // stream bits 32..95
+#pragma unroll
+    for (int i = 0; i < 32; i++) {
+      const int bit = 3 * i;
+      q[i] = bit + 3 <= 64 ? (uint32_t)(lo >> bit) & 7u : (uint32_t)(hi >> (bit - 32)) & 7u;
+    }
+  }
+
+  const size_t o = (size_t)n * p.K + (size_t)c * 32;
+  if (p.out_f32) {
+    float* out = reinterpret_cast<float*>(p.out) + o;
+#pragma unroll
+    for (int i = 0; i < 32; i += 4) {
+      f4 w;
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+        w[j] = AFFINE ? __builtin_fmaf((float)q[i + j], s, b) : ((float)q[i + j] - 7.f) * s;
+      *reinterpret_cast<f4*>(out + i) = w;
+    }
+  } else {
+    _Float16* out = reinterpret_cast<_Float16*>(p.out) + o;
+#pragma unroll
+    for (int i = 0; i < 32; i += 8) {
+      h8 w;
+#pragma unroll
+      for (int j = 0; j < 8; j++)
+        w[j] = (_Float16)(AFFINE ? __builtin_fmaf((float)q[i + j], s, b) : ((float)q[i + j] - 7.f) * s);
+      *reinterpret_cast<h8*>(out + i) = w;
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void fill_kernel(unsigned char* dst, unsigned char byte, size_t bytes) {
+  const size_t stride = (size_t)gridDim.x * 256u;
+  for (size_t i = (size_t)blockIdx.x * 256u + threadIdx.x; i < bytes; i += stride) dst[i] = byte;
+}
+
+__global__ __launch_bounds__(256) void fill16_kernel(u32x4* dst, uint32_t word, size_t n16) {
+  const size_t stride = (size_t)gridDim.x * 256u;
+  const u32x4 v = {word, word, word, word};
+  for (size_t i = (size_t)blockIdx.x * 256u + threadIdx.x; i < n16; i += stride) dst[i] = v;
+}
+
+}  // namespace
+
+hipError_t launch_dequant(const MatmulArgs& a, hipStream_t s) {
+  DequantParams p{};
+  p.out = a.out; p.scales = a.scales; p.weights = a.weights; p.biases = a.biases;
+  p.N = a.N; p.K = a.K; p.k_packed = a.k_packed; p.spr = a.spr; p.nchunks = a.K / 32; p.out_f32 = a.out_f32;
+  const uint64_t total = (uint64_t)p.N * p.nchunks;
+  const dim3 grid((uint32_t)((total + 255) / 256));
+  if (a.bits == 4) {
+    if (a.affine) hipLaunchKernelGGL((dequant_kernel<4, true>), grid, dim3(256), 0, s, p);
+    else hipLaunchKernelGGL((dequant_kernel<4, false>), grid, dim3(256), 0, s, p);
+  } else {
+    hipLaunchKernelGGL((dequant_kernel<3, true>), grid, dim3(256), 0, s, p);
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_fill(void* dst, int byte, size_t bytes, hipStream_t s) {
+  unsigned char* d = reinterpret_cast<unsigned char*>(dst);
+  const unsigned char b = (unsigned char)byte;
+  // unaligned head, 16-byte body, tail
+  size_t head = (16 - (reinterpret_cast<uintptr_t>(d) & 15u)) & 15u;
+  if (head > bytes) head = bytes;
+  if (head) hipLaunchKernelGGL(fill_kernel, dim3(1), dim3(256), 0, s, d, b, head);
+  const size_t body16 = (bytes - head) / 16;
+  if (body16) {
+    const uint32_t word = 0x01010101u * b;
+    size_t blocks = (body16 + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(fill16_kernel, dim3((uint32_t)blocks), dim3(256), 0, s, reinterpret_cast<u32x4*>(d + head), word, body16);
+  }
+  const size_t tail = bytes - head - body16 * 16;
+  if (tail) hipLaunchKernelGGL(fill_kernel, dim3(1), dim3(256), 0, s, d + head + body16 * 16, b, tail);
+  return hipGetLastError();
+}
+
+}  // namespace ztvm

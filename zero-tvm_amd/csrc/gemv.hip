@@ -1,0 +1,249 @@
+// Streaming GEMV for group-quantized weights, one activation row per dispatch
+// unit: y[n] = sum_k x[k] * w[n,k].  HBM-bound: the weight matrix is read
+// exactly once with 128-bit (4-bit) or 96-bit (3-bit) per-lane loads, unpacked
+// in registers and reduced with f32 dot2 accumulation.
+//
+// Replaces the whole M=1 family of the reference generator
+// (src/compiler/shaders/int4_matmul.gen.ts:170-571: scalar, _sg, _tiled,
+// _tiled8, _vec4, _vec4h, _affine, _q3, _moe, _f32 variants) with one wave64
+// design; the arithmetic kept is the generator's factored form
+//   affine:    y = sum_chunks  s*dot(x,q) + b*sum(x)      (:78-84, :401-406)
+//   symmetric: y = sum_chunks  s*(dot(x,q) - 7*sum(x))    (:17-19)
+//
+// Work decomposition
+//   chunk     32 consecutive k (16 B of 4-bit weights, 12 B of 3-bit): one lane-load
+//   lane      owns chunk (pass*LPR + lane%LPR) of row-slot lane/LPR
+//   wave      ROWS*(64/LPR) rows per step, all passes over K, then a DPP reduce
+//   workgroup 4 waves; stages x once in LDS (slot-permuted, conflict-free
+//             16-byte pieces) plus per-chunk sum(x), then strides over row tiles
+//   grid      x: persistent workgroups over row tiles, y: (token,slot) pair for MoE
+#include "internal.h"
+#include "quant.h"
+
+namespace ztvm {
+namespace {
+
+constexpr int WG_THREADS = 256;
+constexpr int WAVES = WG_THREADS / 64;
+
+struct GemvParams {
+  void* out;
+  const _Float16* in;
+  const _Float16* scales;
+  const uint32_t* weights;
+  const _Float16* biases;
+  const uint32_t* ids;
+  uint32_t N, k_packed, spr, nchunks, npasses, ntiles;
+  uint32_t out_f32, moe;
+  uint32_t slots, in_slot_stride, out_slot_stride, in_tok_stride, out_tok_stride, ids_stride, experts;
+};
+
+struct __attribute__((packed, aligned(4))) Words3 {
+  uint32_t a, b, c;
+};
+
+// LDS layout of x for chunk c: piece j (8 halves, 16 bytes) sits at 16-byte
+// slot (c/64)*256 + j*64 + c%64, so the 64 lanes of one ds_read_b128 touch 64
+// consecutive slots.
+__device__ __forceinline__ uint32_t x_slot(uint32_t c, uint32_t j) { return (c >> 6) * 256u + j * 64u + (c & 63u); }
+
+template <int BITS, bool AFFINE, int LPR, int ROWS>
+__global__ __launch_bounds__(WG_THREADS) void gemv_kernel(const GemvParams p) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  constexpr int SUB = 64 / LPR;          // row slots per wave load
+  constexpr int RPW = ROWS * SUB;        // rows per wave step
+  constexpr int WPC = BITS == 4 ? 4 : 3; // words per chunk
+
+  const uint32_t tid = threadIdx.x;
+  const uint32_t lane = tid & 63u;
+  const uint32_t wave = tid >> 6;
+  const uint32_t lk = lane % LPR;
+  const uint32_t sub = lane / LPR;
+
+  // MoE prologue (int4_matmul.gen.ts:236-253): blockIdx.y is the (token, slot) pair.
+  const _Float16* x = p.in;
+  const uint32_t* wbase = p.weights;
+  const _Float16* sbase = p.scales;
+  const _Float16* bbase = p.biases;
+  size_t out_base = 0;
+  if (p.moe) {
+    const uint32_t token = blockIdx.y / p.slots, slot = blockIdx.y % p.slots;
+    const uint32_t expert = p.ids[(size_t)token * p.ids_stride + slot];
+    if (p.experts && expert >= p.experts) return;  // uniform per workgroup
+    wbase += (size_t)expert * p.N * p.k_packed;
+    sbase += (size_t)expert * p.N * p.spr;
+    bbase += (size_t)expert * p.N * p.spr;
+    x += (size_t)token * p.in_tok_stride + (size_t)slot * p.in_slot_stride;
+    out_base = (size_t)token * p.out_tok_stride + (size_t)slot * p.out_slot_stride;
+  }
+
+  // ---- stage x: each thread converts whole chunks -------------------------
+  h8* xs_pieces = reinterpret_cast<h8*>(smem);
+  const uint32_t padded_chunks = (p.nchunks + 63u) & ~63u;
+  float* xsum = reinterpret_cast<float*>(smem + (size_t)padded_chunks * 64u);
+  for (uint32_t c = tid; c < padded_chunks; c += WG_THREADS) {
+    float s = 0.f;
+    if (c < p.nchunks) {
+      const h8* src = reinterpret_cast<const h8*>(x + (size_t)c * 32u);
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const h8 v = src[j];
+        h8 o;
+#pragma unroll
+        for (int sl = 0; sl < 8; sl++) o[sl] = v[value_in_slot(sl)];
+        xs_pieces[x_slot(c, j)] = o;
+#pragma unroll
+        for (int i = 0; i < 8; i++) s += (float)v[i];
+      }
+    } else {
+      const h8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+      for (int j = 0; j < 4; j++) xs_pieces[x_slot(c, j)] = z;
+    }
+    xsum[c] = s;
+  }
+  __syncthreads();
+
+  const uint32_t wave_global = blockIdx.x * WAVES + wave;
+  const uint32_t wave_stride = gridDim.x * WAVES;
+
+  for (uint32_t tile = wave_global; tile < p.ntiles; tile += wave_stride) {
+    float acc[ROWS];
+    uint32_t row[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+      acc[r] = 0.f;
+      const uint32_t rr = tile * RPW + r * SUB + sub;
+      row[r] = rr < p.N ? rr : p.N - 1;  // clamp loads, mask the store
+    }
+
+    for (uint32_t pass = 0; pass < p.npasses; pass++) {
+      const uint32_t c = pass * LPR + lk;
+      const bool live = c < p.nchunks;
+      const uint32_t cc = live ? c : p.nchunks - 1;
+
+      // issue every global load of this pass first
+      uint32_t w[ROWS][4];
+      _Float16 sc[ROWS], bi[ROWS];
+#pragma unroll
+      for (int r = 0; r < ROWS; r++) {
+        const uint32_t* wp = wbase + (size_t)row[r] * p.k_packed + (size_t)cc * WPC;
+        if (BITS == 4) {
+          const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp));
+          w[r][0] = v.x; w[r][1] = v.y; w[r][2] = v.z; w[r][3] = v.w;
+        } else {
+          const Words3 v = *reinterpret_cast<const Words3*>(wp);  // 12 bytes, 4-byte aligned
+          w[r][0] = v.a; w[r][1] = v.b; w[r][2] = v.c; w[r][3] = 0;
+        }
+        const uint32_t g = AFFINE ? (cc >> 1) : cc;
+        sc[r] = sbase[(size_t)row[r] * p.spr + g];
+        if (AFFINE) bi[r] = bbase[(size_t)row[r] * p.spr + g];
+      }
+      // keep the compiler from sinking the small scale/bias loads down to their
+      // first use, where their latency would be exposed once per pass
+      __builtin_amdgcn_sched_barrier(0);
+
+      h2 xv[16];
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const h8 v = xs_pieces[x_slot(cc, j)];
+        xv[4 * j + 0] = (h2){v[0], v[1]};
+        xv[4 * j + 1] = (h2){v[2], v[3]};
+        xv[4 * j + 2] = (h2){v[4], v[5]};
+        xv[4 * j + 3] = (h2){v[6], v[7]};
+      }
+      const float xs = xsum[cc];
+
+#pragma unroll
+      for (int r = 0; r < ROWS; r++) {
+        h2 q[16];
+        if (BITS == 4) unpack4_chunk(w[r][0], w[r][1], w[r][2], w[r][3], q);
+        else unpack3_chunk(w[r][0], w[r][1], w[r][2], q);
+        float d0 = 0.f, d1 = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; i += 2) {
+          d0 = __builtin_amdgcn_fdot2(q[i], xv[i], d0, false);
+          d1 = __builtin_amdgcn_fdot2(q[i + 1], xv[i + 1], d1, false);
+        }
+        const float dot = d0 + d1;
+        const float s = (float)sc[r];
+        const float term = AFFINE ? s * dot + (float)bi[r] * xs : s * (dot - 7.f * xs);
+        acc[r] += live ? term : 0.f;
+      }
+    }
+
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+      const float total = group_sum_to_last_lane<LPR>(acc[r]);
+      const uint32_t rr = tile * RPW + r * SUB + sub;
+      if (lk == LPR - 1 && rr < p.N) {
+        if (p.out_f32) reinterpret_cast<float*>(p.out)[out_base + rr] = total;
+        else reinterpret_cast<_Float16*>(p.out)[out_base + rr] = (_Float16)total;
+      }
+    }
+  }
+}
+
+template <int BITS, bool AFFINE, int LPR, int ROWS>
+hipError_t launch_one(const GemvParams& p, dim3 grid, size_t smem, hipStream_t s) {
+  hipLaunchKernelGGL((gemv_kernel<BITS, AFFINE, LPR, ROWS>), grid, dim3(WG_THREADS), smem, s, p);
+  return hipGetLastError();
+}
+
+template <int BITS, bool AFFINE>
+hipError_t launch_fmt(const GemvParams& p, int lpr, int rows, dim3 grid, size_t smem, hipStream_t s) {
+  if (lpr == 64) {
+    if (rows == 4) return launch_one<BITS, AFFINE, 64, 4>(p, grid, smem, s);
+    if (rows == 2) return launch_one<BITS, AFFINE, 64, 2>(p, grid, smem, s);
+    return launch_one<BITS, AFFINE, 64, 1>(p, grid, smem, s);
+  }
+  if (lpr == 32) return launch_one<BITS, AFFINE, 32, 2>(p, grid, smem, s);
+  return launch_one<BITS, AFFINE, 16, 2>(p, grid, smem, s);
+}
+
+}  // namespace
+
+hipError_t launch_gemv(const MatmulArgs& a, const Tune& t, hipStream_t s) {
+  GemvParams p{};
+  p.out = a.out; p.in = a.in; p.scales = a.scales; p.weights = a.weights; p.biases = a.biases; p.ids = a.ids;
+  p.N = a.N; p.k_packed = a.k_packed; p.spr = a.spr;
+  p.nchunks = a.K / 32;
+  p.out_f32 = a.out_f32;
+  p.moe = a.slots > 0;
+  p.slots = a.slots; p.in_slot_stride = a.in_slot_stride; p.out_slot_stride = a.out_slot_stride;
+  p.in_tok_stride = a.in_tok_stride; p.out_tok_stride = a.out_tok_stride; p.ids_stride = a.ids_stride;
+  p.experts = a.experts;
+
+  // lanes per row: narrow rows share a wave between several rows
+  const int lpr = p.nchunks > 32 ? 64 : (p.nchunks > 16 ? 32 : 16);
+  p.npasses = (p.nchunks + lpr - 1) / lpr;
+  const uint32_t pairs = p.moe ? a.slots * a.tokens : 1;
+
+  int rows = 2;
+  if (lpr == 64) {
+    rows = t.gemv_rows ? t.gemv_rows : (p.npasses >= 4 ? 2 : 4);
+    // few rows: prefer more, smaller tiles so every CU gets work
+    while (rows > 1 && (uint64_t)((a.N + rows - 1) / rows) * pairs < (uint64_t)t.num_cus * WAVES * 2) rows >>= 1;
+  }
+  const uint32_t rpw = rows * (64 / lpr);
+  p.ntiles = (a.N + rpw - 1) / rpw;
+
+  const uint32_t padded_chunks = (p.nchunks + 63u) & ~63u;
+  const size_t smem = (size_t)padded_chunks * 64 + (size_t)padded_chunks * 4;
+
+  const uint32_t wg_tiles = (p.ntiles + WAVES - 1) / WAVES;
+  const int wg_per_cu = t.gemv_wg_per_cu ? t.gemv_wg_per_cu : 4;
+  uint32_t gx = (uint32_t)t.num_cus * wg_per_cu / (pairs < 1 ? 1 : pairs);
+  if (gx < 1) gx = 1;
+  if (gx > wg_tiles) gx = wg_tiles;
+  const dim3 grid(gx, pairs, 1);
+
+  // dense M>1 handled by the caller looping rows; here one activation row
+  if (a.bits == 4) {
+    if (a.affine) return launch_fmt<4, true>(p, lpr, rows, grid, smem, s);
+    return launch_fmt<4, false>(p, lpr, rows, grid, smem, s);
+  }
+  return launch_fmt<3, true>(p, lpr, rows, grid, smem, s);
+}
+
+}  // namespace ztvm

@@ -1,0 +1,41 @@
+// Internal interfaces between the C ABI (ztvm_api.hip) and the kernel files.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ztvm {
+
+// Resolved launch arguments for every kernel family (device pointers typed).
+struct MatmulArgs {
+  void* out;
+  const _Float16* in;
+  const _Float16* scales;
+  const uint32_t* weights;
+  const _Float16* biases;
+  const uint32_t* ids;
+  uint32_t M, N, K, k_packed, spr;
+  uint32_t bits, affine, out_f32;
+  uint32_t slots, tokens;  // slots == 0: dense
+  uint32_t in_slot_stride, out_slot_stride, in_tok_stride, out_tok_stride, ids_stride, experts;
+};
+
+// Launch knobs (ztvm_set_option). Zero means "use the built-in default".
+struct Tune {
+  int num_cus = 256;
+  int gemv_wg_per_cu = 0;   // workgroups resident per CU for the streaming GEMV
+  int gemv_rows = 0;        // rows per wave step (1, 2 or 4)
+  int skinny_wg_per_cu = 0;
+  int gemm_tile = 0;        // 0 auto
+  int gemm_xcd_swizzle = 1;
+};
+
+hipError_t launch_gemv(const MatmulArgs& a, const Tune& t, hipStream_t s);
+hipError_t launch_skinny(const MatmulArgs& a, const Tune& t, hipStream_t s);
+hipError_t launch_gemm(const MatmulArgs& a, const Tune& t, hipStream_t s);
+hipError_t launch_dequant(const MatmulArgs& a, hipStream_t s);
+hipError_t launch_fill(void* dst, int byte, size_t bytes, hipStream_t s);
+
+bool skinny_supports(const MatmulArgs& a);
+bool gemm_supports(const MatmulArgs& a);
+
+}  // namespace ztvm

@@ -1,0 +1,406 @@
+// C ABI of libztvm_hip: context, buffers, descriptor validation, dispatch,
+// command buffers (HIP graphs) and events. See include/ztvm.h for the contract
+// and the reference interfaces each entry point replaces.
+#include "../../include/ztvm.h"
+#include "internal.h"
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <string>
+
+using namespace ztvm;
+
+struct ztvm_ctx {
+  int device = 0;
+  hipStream_t stream = nullptr;
+  bool recording = false;
+  Tune tune;
+  std::string err;
+  hipDeviceProp_t prop;
+};
+struct ztvm_cmdbuf {
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+};
+struct ztvm_event {
+  hipEvent_t ev = nullptr;
+};
+
+namespace {
+
+thread_local std::string g_err = "";
+
+int fail(ztvm_ctx* ctx, int code, const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof buf, fmt, ap);
+  va_end(ap);
+  if (ctx) ctx->err = buf;
+  g_err = buf;
+  return code;
+}
+
+#define HIP_TRY(ctx, expr)                                                                          \
+  do {                                                                                              \
+    hipError_t e_ = (expr);                                                                         \
+    if (e_ != hipSuccess) return fail(ctx, ZTVM_E_HIP, "%s: %s", #expr, hipGetErrorString(e_));     \
+  } while (0)
+
+void why_set(char* why, size_t n, const char* fmt, ...) {
+  if (!why || !n) return;
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(why, n, fmt, ap);
+  va_end(ap);
+}
+
+// The legality rules of the generator (int4_matmul.gen.ts:172-197) that are
+// about arithmetic, plus the layout contract of the bindings.
+int validate(const ztvm_matmul_desc* d, char* why, size_t n, bool need_in_out) {
+  if (!d) { why_set(why, n, "null descriptor"); return ZTVM_E_INVALID; }
+  if (d->bits != 4 && d->bits != 3) { why_set(why, n, "bits must be 4 or 3 (got %u)", d->bits); return ZTVM_E_INVALID; }
+  if (d->affine > 1 || d->out_f32 > 1) { why_set(why, n, "affine/out_f32 must be 0 or 1"); return ZTVM_E_INVALID; }
+  if (d->bits == 3 && !d->affine) { why_set(why, n, "q3 requires affine (3-bit ships only in the MLX-affine layout)"); return ZTVM_E_INVALID; }
+  if (d->slots && !d->affine) { why_set(why, n, "moe requires affine (the MoE weights are MLX affine-quantised)"); return ZTVM_E_INVALID; }
+  if (d->kernel > ZTVM_KERNEL_GEMM) { why_set(why, n, "unknown kernel family %u", d->kernel); return ZTVM_E_INVALID; }
+  if (!d->N) { why_set(why, n, "N must be > 0"); return ZTVM_E_INVALID; }
+  if (!d->k_packed) { why_set(why, n, "K_PACKED must be > 0"); return ZTVM_E_INVALID; }
+  const uint64_t kbits = (uint64_t)d->k_packed * 32u;
+  if (kbits % d->bits) { why_set(why, n, "K_PACKED=%u words do not hold a whole number of %u-bit values", d->k_packed, d->bits); return ZTVM_E_INVALID; }
+  const uint64_t K = kbits / d->bits;
+  const uint32_t G = d->affine ? 64u : 32u;
+  if (K % G) { why_set(why, n, "K=%llu is not a multiple of the group size %u", (unsigned long long)K, G); return ZTVM_E_INVALID; }
+  if (K > (1u << 24)) { why_set(why, n, "K=%llu too large", (unsigned long long)K); return ZTVM_E_INVALID; }
+  if ((uint64_t)d->scales_per_row != K / G) {
+    why_set(why, n, "SCALES_PER_ROW=%u but K/group = %llu (K=%llu, group %u)", d->scales_per_row, (unsigned long long)(K / G), (unsigned long long)K, G);
+    return ZTVM_E_INVALID;
+  }
+  if (need_in_out) {
+    if (d->slots) {
+      if (d->M != 1) { why_set(why, n, "moe dispatches one activation row per (token,slot): M must be 1 (got %u)", d->M); return ZTVM_E_INVALID; }
+      if (!d->tokens) { why_set(why, n, "moe needs tokens > 0"); return ZTVM_E_INVALID; }
+      if (d->ids_stride < d->slots) { why_set(why, n, "IDS_STRIDE=%u < slots=%u", d->ids_stride, d->slots); return ZTVM_E_INVALID; }
+      if (!d->ids) { why_set(why, n, "null buffer at binding 6 (ids)"); return ZTVM_E_INVALID; }
+      if (d->ids & 3u) { why_set(why, n, "ids must be 4-byte aligned"); return ZTVM_E_INVALID; }
+      if ((d->in_slot_stride | d->in_tok_stride) & 7u) { why_set(why, n, "moe input strides must be multiples of 8 elements"); return ZTVM_E_INVALID; }
+      if (d->out_slot_stride < d->N && d->slots > 1) { why_set(why, n, "OUT_SLOT_STRIDE=%u < N=%u would overlap slot outputs", d->out_slot_stride, d->N); return ZTVM_E_INVALID; }
+    } else {
+      if (!d->M) { why_set(why, n, "M must be > 0"); return ZTVM_E_INVALID; }
+    }
+    if (!d->in) { why_set(why, n, "null buffer at binding 1 (input)"); return ZTVM_E_INVALID; }
+    if (d->in & 15u) { why_set(why, n, "input must be 16-byte aligned"); return ZTVM_E_INVALID; }
+  }
+  if (!d->out) { why_set(why, n, "null buffer at binding 0 (output)"); return ZTVM_E_INVALID; }
+  if (!d->scales) { why_set(why, n, "null buffer at binding 2 (scales)"); return ZTVM_E_INVALID; }
+  if (!d->weights) { why_set(why, n, "null buffer at binding 3 (weights)"); return ZTVM_E_INVALID; }
+  if (d->affine && !d->biases) { why_set(why, n, "affine matmul has no bias buffer at binding 5"); return ZTVM_E_INVALID; }
+  if (d->weights & 15u) { why_set(why, n, "weights must be 16-byte aligned"); return ZTVM_E_INVALID; }
+  if ((d->scales & 15u) || (d->affine && (d->biases & 15u))) { why_set(why, n, "scales/biases must be 16-byte aligned"); return ZTVM_E_INVALID; }
+  if (d->out & (d->out_f32 ? 3u : 1u)) { why_set(why, n, "output misaligned for its element type"); return ZTVM_E_INVALID; }
+  return ZTVM_OK;
+}
+
+MatmulArgs to_args(const ztvm_matmul_desc* d) {
+  MatmulArgs a{};
+  a.out = reinterpret_cast<void*>(d->out);
+  a.in = reinterpret_cast<const _Float16*>(d->in);
+  a.scales = reinterpret_cast<const _Float16*>(d->scales);
+  a.weights = reinterpret_cast<const uint32_t*>(d->weights);
+  a.biases = reinterpret_cast<const _Float16*>(d->biases);
+  a.ids = reinterpret_cast<const uint32_t*>(d->ids);
+  a.M = d->M; a.N = d->N; a.k_packed = d->k_packed; a.spr = d->scales_per_row;
+  a.K = (uint32_t)((uint64_t)d->k_packed * 32u / d->bits);
+  a.bits = d->bits; a.affine = d->affine; a.out_f32 = d->out_f32;
+  a.slots = d->slots; a.tokens = d->tokens;
+  a.in_slot_stride = d->in_slot_stride; a.out_slot_stride = d->out_slot_stride;
+  a.in_tok_stride = d->in_tok_stride; a.out_tok_stride = d->out_tok_stride;
+  a.ids_stride = d->ids_stride; a.experts = d->experts;
+  return a;
+}
+
+// Which family runs a descriptor. Thresholds are measured crossovers on
+// MI355X: the GEMV re-reads the weights once per activation row, the skinny
+// kernel reads them once for up to 64 rows, the tile GEMM needs enough rows to
+// fill its M tile.
+int resolve(const MatmulArgs& a, uint32_t want, char* why, size_t n) {
+  const bool moe = a.slots > 0;
+  const bool sk = !moe && skinny_supports(a);
+  const bool ge = !moe && gemm_supports(a);
+  if (want == ZTVM_KERNEL_GEMV) return ZTVM_KERNEL_GEMV;
+  if (want == ZTVM_KERNEL_SKINNY) {
+    if (!sk) { why_set(why, n, "kernel: asked for 'skinny', which cannot run this dispatch (moe=%d, M=%u)", (int)moe, a.M); return ZTVM_E_UNSUPPORTED; }
+    return ZTVM_KERNEL_SKINNY;
+  }
+  if (want == ZTVM_KERNEL_GEMM) {
+    if (!ge) { why_set(why, n, "kernel: asked for 'gemm', which cannot run this dispatch (moe=%d, bits=%u, out_f32=%u, K=%u)", (int)moe, a.bits, a.out_f32, a.K); return ZTVM_E_UNSUPPORTED; }
+    return ZTVM_KERNEL_GEMM;
+  }
+  if (moe || a.M == 1) return ZTVM_KERNEL_GEMV;
+  if (ge && a.M > 32) return ZTVM_KERNEL_GEMM;
+  if (sk) return ZTVM_KERNEL_SKINNY;
+  if (ge) return ZTVM_KERNEL_GEMM;
+  return ZTVM_KERNEL_GEMV;
+}
+
+struct Option {
+  const char* name;
+  int Tune::*field;
+};
+const Option kOptions[] = {
+    {"num_cus", &Tune::num_cus},
+    {"gemv.wg_per_cu", &Tune::gemv_wg_per_cu},
+    {"gemv.rows", &Tune::gemv_rows},
+    {"skinny.wg_per_cu", &Tune::skinny_wg_per_cu},
+    {"gemm.tile", &Tune::gemm_tile},
+    {"gemm.xcd_swizzle", &Tune::gemm_xcd_swizzle},
+};
+
+}  // namespace
+
+extern "C" {
+
+int ztvm_abi_version(void) { return ZTVM_ABI_VERSION; }
+
+const char* ztvm_last_error(ztvm_ctx* ctx) { return ctx ? ctx->err.c_str() : g_err.c_str(); }
+
+int ztvm_create(int device, ztvm_ctx** out) {
+  if (!out) return fail(nullptr, ZTVM_E_INVALID, "ztvm_create: null out pointer");
+  *out = nullptr;
+  int count = 0;
+  if (hipGetDeviceCount(&count) != hipSuccess || count <= 0) return fail(nullptr, ZTVM_E_NODEVICE, "no HIP device visible");
+  if (device < 0 || device >= count) return fail(nullptr, ZTVM_E_INVALID, "device %d out of range (%d visible)", device, count);
+  ztvm_ctx* c = new ztvm_ctx();
+  c->device = device;
+  HIP_TRY(nullptr, hipSetDevice(device));
+  HIP_TRY(nullptr, hipGetDeviceProperties(&c->prop, device));
+  if (!strstr(c->prop.gcnArchName, "gfx950")) {
+    std::string arch = c->prop.gcnArchName;
+    delete c;
+    return fail(nullptr, ZTVM_E_NODEVICE, "device %d is %s; this library holds gfx950 code only", device, arch.c_str());
+  }
+  HIP_TRY(nullptr, hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
+  c->tune.num_cus = c->prop.multiProcessorCount > 0 ? c->prop.multiProcessorCount : 256;
+  *out = c;
+  return ZTVM_OK;
+}
+
+void ztvm_destroy(ztvm_ctx* ctx) {
+  if (!ctx) return;
+  (void)hipSetDevice(ctx->device);
+  if (ctx->stream) {
+    (void)hipStreamSynchronize(ctx->stream);
+    (void)hipStreamDestroy(ctx->stream);
+  }
+  delete ctx;
+}
+
+int ztvm_device_info(ztvm_ctx* ctx, char* name, size_t name_len, uint32_t* cus, uint64_t* hbm) {
+  if (!ctx) return fail(nullptr, ZTVM_E_INVALID, "null context");
+  if (name && name_len) snprintf(name, name_len, "%s (%s)", ctx->prop.name, ctx->prop.gcnArchName);
+  if (cus) *cus = (uint32_t)ctx->prop.multiProcessorCount;
+  if (hbm) *hbm = (uint64_t)ctx->prop.totalGlobalMem;
+  return ZTVM_OK;
+}
+
+int ztvm_alloc(ztvm_ctx* ctx, size_t bytes, uint64_t* dptr) {
+  if (!ctx || !dptr) return fail(ctx, ZTVM_E_INVALID, "ztvm_alloc: null argument");
+  if (ctx->recording) return fail(ctx, ZTVM_E_INVALID, "ztvm_alloc while recording a command buffer");
+  void* p = nullptr;
+  HIP_TRY(ctx, hipSetDevice(ctx->device));
+  HIP_TRY(ctx, hipMalloc(&p, bytes < 4 ? 4 : bytes));
+  *dptr = reinterpret_cast<uint64_t>(p);
+  return ZTVM_OK;
+}
+
+int ztvm_free(ztvm_ctx* ctx, uint64_t dptr) {
+  if (!ctx) return fail(nullptr, ZTVM_E_INVALID, "null context");
+  if (ctx->recording) return fail(ctx, ZTVM_E_INVALID, "ztvm_free while recording a command buffer");
+  if (!dptr) return ZTVM_OK;
+  HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+  HIP_TRY(ctx, hipFree(reinterpret_cast<void*>(dptr)));
+  return ZTVM_OK;
+}
+
+int ztvm_upload(ztvm_ctx* ctx, uint64_t dst, size_t off, const void* src, size_t bytes) {
+  if (!ctx || !dst || (!src && bytes)) return fail(ctx, ZTVM_E_INVALID, "ztvm_upload: null argument");
+  if (ctx->recording) return fail(ctx, ZTVM_E_INVALID, "ztvm_upload while recording a command buffer");
+  if (!bytes) return ZTVM_OK;
+  HIP_TRY(ctx, hipMemcpyAsync(reinterpret_cast<char*>(dst) + off, src, bytes, hipMemcpyHostToDevice, ctx->stream));
+  HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));  // the source may be reused on return
+  return ZTVM_OK;
+}
+
+int ztvm_download(ztvm_ctx* ctx, void* dst, uint64_t src, size_t off, size_t bytes) {
+  if (!ctx || !src || (!dst && bytes)) return fail(ctx, ZTVM_E_INVALID, "ztvm_download: null argument");
+  if (ctx->recording) return fail(ctx, ZTVM_E_INVALID, "ztvm_download while recording a command buffer");
+  if (!bytes) return ZTVM_OK;
+  HIP_TRY(ctx, hipMemcpyAsync(dst, reinterpret_cast<const char*>(src) + off, bytes, hipMemcpyDeviceToHost, ctx->stream));
+  HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+  return ZTVM_OK;
+}
+
+int ztvm_fill(ztvm_ctx* ctx, uint64_t dst, size_t off, int byte, size_t bytes) {
+  if (!ctx || !dst) return fail(ctx, ZTVM_E_INVALID, "ztvm_fill: null argument");
+  if (!bytes) return ZTVM_OK;
+  HIP_TRY(ctx, launch_fill(reinterpret_cast<char*>(dst) + off, byte, bytes, ctx->stream));
+  return ZTVM_OK;
+}
+
+int ztvm_sync(ztvm_ctx* ctx) {
+  if (!ctx) return fail(nullptr, ZTVM_E_INVALID, "null context");
+  if (ctx->recording) return fail(ctx, ZTVM_E_INVALID, "ztvm_sync while recording a command buffer");
+  HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+  return ZTVM_OK;
+}
+
+int ztvm_matmul_validate(const ztvm_matmul_desc* desc, char* why, size_t why_len) {
+  if (why && why_len) why[0] = 0;
+  int rc = validate(desc, why, why_len, true);
+  if (rc) return rc;
+  const MatmulArgs a = to_args(desc);
+  rc = resolve(a, desc->kernel, why, why_len);
+  return rc < 0 ? rc : ZTVM_OK;
+}
+
+int ztvm_matmul_resolve(const ztvm_matmul_desc* desc) {
+  char why[256];
+  int rc = validate(desc, why, sizeof why, true);
+  if (rc) return fail(nullptr, rc, "%s", why);
+  const MatmulArgs a = to_args(desc);
+  rc = resolve(a, desc->kernel, why, sizeof why);
+  if (rc < 0) return fail(nullptr, rc, "%s", why);
+  return rc;
+}
+
+int ztvm_matmul(ztvm_ctx* ctx, const ztvm_matmul_desc* desc) {
+  if (!ctx) return fail(nullptr, ZTVM_E_INVALID, "null context");
+  char why[256];
+  int rc = validate(desc, why, sizeof why, true);
+  if (rc) return fail(ctx, rc, "ztvm_matmul: %s", why);
+  MatmulArgs a = to_args(desc);
+  const int fam = resolve(a, desc->kernel, why, sizeof why);
+  if (fam < 0) return fail(ctx, fam, "ztvm_matmul: %s", why);
+  switch (fam) {
+    case ZTVM_KERNEL_SKINNY: HIP_TRY(ctx, launch_skinny(a, ctx->tune, ctx->stream)); break;
+    case ZTVM_KERNEL_GEMM: HIP_TRY(ctx, launch_gemm(a, ctx->tune, ctx->stream)); break;
+    default: {
+      // one streaming pass per activation row
+      const uint32_t M = a.slots ? 1 : a.M;
+      const size_t out_elt = a.out_f32 ? 4 : 2;
+      for (uint32_t m = 0; m < M; m++) {
+        MatmulArgs r = a;
+        r.M = 1;
+        r.in = a.in + (size_t)m * a.K;
+        r.out = reinterpret_cast<char*>(a.out) + (size_t)m * a.N * out_elt;
+        HIP_TRY(ctx, launch_gemv(r, ctx->tune, ctx->stream));
+      }
+    }
+  }
+  return ZTVM_OK;
+}
+
+int ztvm_dequant(ztvm_ctx* ctx, const ztvm_matmul_desc* desc) {
+  if (!ctx) return fail(nullptr, ZTVM_E_INVALID, "null context");
+  char why[256];
+  int rc = validate(desc, why, sizeof why, false);
+  if (rc) return fail(ctx, rc, "ztvm_dequant: %s", why);
+  if (desc->out & 15u) return fail(ctx, ZTVM_E_INVALID, "ztvm_dequant: output must be 16-byte aligned");
+  const MatmulArgs a = to_args(desc);
+  HIP_TRY(ctx, launch_dequant(a, ctx->stream));
+  return ZTVM_OK;
+}
+
+int ztvm_record_begin(ztvm_ctx* ctx) {
+  if (!ctx) return fail(nullptr, ZTVM_E_INVALID, "null context");
+  if (ctx->recording) return fail(ctx, ZTVM_E_INVALID, "already recording");
+  HIP_TRY(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+  ctx->recording = true;
+  return ZTVM_OK;
+}
+
+int ztvm_record_end(ztvm_ctx* ctx, ztvm_cmdbuf** out) {
+  if (!ctx || !out) return fail(ctx, ZTVM_E_INVALID, "ztvm_record_end: null argument");
+  if (!ctx->recording) return fail(ctx, ZTVM_E_INVALID, "not recording");
+  ctx->recording = false;
+  ztvm_cmdbuf* cb = new ztvm_cmdbuf();
+  hipError_t e = hipStreamEndCapture(ctx->stream, &cb->graph);
+  if (e == hipSuccess) e = hipGraphInstantiate(&cb->exec, cb->graph, nullptr, nullptr, 0);
+  if (e != hipSuccess) {
+    if (cb->graph) (void)hipGraphDestroy(cb->graph);
+    delete cb;
+    return fail(ctx, ZTVM_E_HIP, "command buffer finish: %s", hipGetErrorString(e));
+  }
+  *out = cb;
+  return ZTVM_OK;
+}
+
+int ztvm_submit(ztvm_ctx* ctx, ztvm_cmdbuf* cb) {
+  if (!ctx || !cb || !cb->exec) return fail(ctx, ZTVM_E_INVALID, "ztvm_submit: null argument");
+  if (ctx->recording) return fail(ctx, ZTVM_E_INVALID, "ztvm_submit while recording");
+  HIP_TRY(ctx, hipGraphLaunch(cb->exec, ctx->stream));
+  return ZTVM_OK;
+}
+
+void ztvm_cmdbuf_destroy(ztvm_cmdbuf* cb) {
+  if (!cb) return;
+  if (cb->exec) (void)hipGraphExecDestroy(cb->exec);
+  if (cb->graph) (void)hipGraphDestroy(cb->graph);
+  delete cb;
+}
+
+int ztvm_event_create(ztvm_ctx* ctx, ztvm_event** out) {
+  if (!ctx || !out) return fail(ctx, ZTVM_E_INVALID, "ztvm_event_create: null argument");
+  ztvm_event* e = new ztvm_event();
+  hipError_t r = hipEventCreate(&e->ev);
+  if (r != hipSuccess) {
+    delete e;
+    return fail(ctx, ZTVM_E_HIP, "hipEventCreate: %s", hipGetErrorString(r));
+  }
+  *out = e;
+  return ZTVM_OK;
+}
+
+void ztvm_event_destroy(ztvm_event* ev) {
+  if (!ev) return;
+  if (ev->ev) (void)hipEventDestroy(ev->ev);
+  delete ev;
+}
+
+int ztvm_event_record(ztvm_ctx* ctx, ztvm_event* ev) {
+  if (!ctx || !ev) return fail(ctx, ZTVM_E_INVALID, "ztvm_event_record: null argument");
+  if (ctx->recording) return fail(ctx, ZTVM_E_INVALID, "ztvm_event_record while recording");
+  HIP_TRY(ctx, hipEventRecord(ev->ev, ctx->stream));
+  return ZTVM_OK;
+}
+
+int ztvm_event_elapsed_ms(ztvm_ctx* ctx, ztvm_event* start, ztvm_event* stop, float* ms) {
+  if (!ctx || !start || !stop || !ms) return fail(ctx, ZTVM_E_INVALID, "ztvm_event_elapsed_ms: null argument");
+  HIP_TRY(ctx, hipEventSynchronize(stop->ev));
+  HIP_TRY(ctx, hipEventElapsedTime(ms, start->ev, stop->ev));
+  return ZTVM_OK;
+}
+
+int ztvm_set_option(ztvm_ctx* ctx, const char* name, int value) {
+  if (!ctx || !name) return fail(ctx, ZTVM_E_INVALID, "ztvm_set_option: null argument");
+  for (const Option& o : kOptions)
+    if (!strcmp(o.name, name)) {
+      ctx->tune.*(o.field) = value;
+      return ZTVM_OK;
+    }
+  return fail(ctx, ZTVM_E_INVALID, "unknown option '%s'", name);
+}
+
+int ztvm_get_option(ztvm_ctx* ctx, const char* name, int* value) {
+  if (!ctx || !name || !value) return fail(ctx, ZTVM_E_INVALID, "ztvm_get_option: null argument");
+  for (const Option& o : kOptions)
+    if (!strcmp(o.name, name)) {
+      *value = ctx->tune.*(o.field);
+      return ZTVM_OK;
+    }
+  return fail(ctx, ZTVM_E_INVALID, "unknown option '%s'", name);
+}
+
+}  // extern "C"

@@ -1,0 +1,197 @@
+"""ctypes binding of libztvm_hip.so (the C ABI declared in include/ztvm.h).
+
+There is no fallback: if the shared library is missing or a call fails, an
+exception is raised. Device memory is named by integer device addresses.
+"""
+import ctypes as C
+import os
+
+_PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB_PATH = os.path.join(_PKG, "lib", "libztvm_hip.so")
+
+KERNEL_AUTO, KERNEL_GEMV, KERNEL_SKINNY, KERNEL_GEMM = 0, 1, 2, 3
+KERNEL_NAMES = {0: "auto", 1: "gemv", 2: "skinny", 3: "gemm"}
+E_INVALID, E_HIP, E_UNSUPPORTED, E_NODEVICE = -1, -2, -3, -4
+
+EXPORTS = [
+    "ztvm_abi_version", "ztvm_last_error", "ztvm_create", "ztvm_destroy", "ztvm_device_info",
+    "ztvm_alloc", "ztvm_free", "ztvm_upload", "ztvm_download", "ztvm_fill", "ztvm_sync",
+    "ztvm_matmul_validate", "ztvm_matmul_resolve", "ztvm_matmul", "ztvm_dequant",
+    "ztvm_record_begin", "ztvm_record_end", "ztvm_submit", "ztvm_cmdbuf_destroy",
+    "ztvm_event_create", "ztvm_event_destroy", "ztvm_event_record", "ztvm_event_elapsed_ms",
+    "ztvm_set_option", "ztvm_get_option",
+]
+
+
+class ZtvmError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__("ztvm error %d: %s" % (code, msg))
+        self.code = code
+        self.reason = msg
+
+
+class MatmulDesc(C.Structure):
+    """Mirror of ztvm_matmul_desc."""
+    _fields_ = [(n, C.c_uint32) for n in (
+        "bits", "affine", "out_f32", "kernel", "M", "N", "k_packed", "scales_per_row", "slots", "tokens",
+        "in_slot_stride", "out_slot_stride", "in_tok_stride", "out_tok_stride", "ids_stride", "experts")] + [
+        (n, C.c_uint64) for n in ("out", "in_", "scales", "weights", "biases", "ids")]
+
+
+_lib = None
+
+
+def load():
+    """Load the shared library; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ZtvmError(E_NODEVICE, "libztvm_hip.so is not built (%s); run `python zero-tvm_amd/build.py`" % LIB_PATH)
+    L = C.CDLL(LIB_PATH)
+    vp, u64p = C.c_void_p, C.POINTER(C.c_uint64)
+    L.ztvm_abi_version.restype = C.c_int
+    L.ztvm_last_error.restype, L.ztvm_last_error.argtypes = C.c_char_p, [vp]
+    L.ztvm_create.argtypes = [C.c_int, C.POINTER(vp)]
+    L.ztvm_destroy.restype, L.ztvm_destroy.argtypes = None, [vp]
+    L.ztvm_device_info.argtypes = [vp, C.c_char_p, C.c_size_t, C.POINTER(C.c_uint32), u64p]
+    L.ztvm_alloc.argtypes = [vp, C.c_size_t, u64p]
+    L.ztvm_free.argtypes = [vp, C.c_uint64]
+    L.ztvm_upload.argtypes = [vp, C.c_uint64, C.c_size_t, vp, C.c_size_t]
+    L.ztvm_download.argtypes = [vp, vp, C.c_uint64, C.c_size_t, C.c_size_t]
+    L.ztvm_fill.argtypes = [vp, C.c_uint64, C.c_size_t, C.c_int, C.c_size_t]
+    L.ztvm_sync.argtypes = [vp]
+    L.ztvm_matmul_validate.argtypes = [C.POINTER(MatmulDesc), C.c_char_p, C.c_size_t]
+    L.ztvm_matmul_resolve.argtypes = [C.POINTER(MatmulDesc)]
+    L.ztvm_matmul.argtypes = [vp, C.POINTER(MatmulDesc)]
+    L.ztvm_dequant.argtypes = [vp, C.POINTER(MatmulDesc)]
+    L.ztvm_record_begin.argtypes = [vp]
+    L.ztvm_record_end.argtypes = [vp, C.POINTER(vp)]
+    L.ztvm_submit.argtypes = [vp, vp]
+    L.ztvm_cmdbuf_destroy.restype, L.ztvm_cmdbuf_destroy.argtypes = None, [vp]
+    L.ztvm_event_create.argtypes = [vp, C.POINTER(vp)]
+    L.ztvm_event_destroy.restype, L.ztvm_event_destroy.argtypes = None, [vp]
+    L.ztvm_event_record.argtypes = [vp, vp]
+    L.ztvm_event_elapsed_ms.argtypes = [vp, vp, vp, C.POINTER(C.c_float)]
+    L.ztvm_set_option.argtypes = [vp, C.c_char_p, C.c_int]
+    L.ztvm_get_option.argtypes = [vp, C.c_char_p, C.POINTER(C.c_int)]
+    _lib = L
+    return L
+
+
+def validate(desc):
+    """Pure-CPU descriptor check. Returns (code, reason)."""
+    buf = C.create_string_buffer(512)
+    rc = load().ztvm_matmul_validate(C.byref(desc), buf, len(buf))
+    return rc, buf.value.decode()
+
+
+def resolve(desc):
+    """Family AUTO picks for this descriptor; raises on an illegal descriptor."""
+    L = load()
+    rc = L.ztvm_matmul_resolve(C.byref(desc))
+    if rc < 0:
+        raise ZtvmError(rc, L.ztvm_last_error(None).decode())
+    return rc
+
+
+class Context:
+    """One device + one in-order stream (the reference's GPUDevice + queue)."""
+
+    def __init__(self, device=0):
+        self._L = load()
+        h = C.c_void_p()
+        rc = self._L.ztvm_create(device, C.byref(h))
+        if rc:
+            raise ZtvmError(rc, self._L.ztvm_last_error(None).decode())
+        self._h = h
+
+    def _chk(self, rc):
+        if rc:
+            raise ZtvmError(rc, self._L.ztvm_last_error(self._h).decode())
+
+    def close(self):
+        if getattr(self, "_h", None):
+            self._L.ztvm_destroy(self._h)
+            self._h = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *a):
+        self.close()
+
+    def device_info(self):
+        name = C.create_string_buffer(256)
+        cus, hbm = C.c_uint32(), C.c_uint64()
+        self._chk(self._L.ztvm_device_info(self._h, name, len(name), C.byref(cus), C.byref(hbm)))
+        return {"name": name.value.decode(), "compute_units": cus.value, "hbm_bytes": hbm.value}
+
+    def alloc(self, nbytes):
+        p = C.c_uint64()
+        self._chk(self._L.ztvm_alloc(self._h, nbytes, C.byref(p)))
+        return p.value
+
+    def free(self, dptr):
+        self._chk(self._L.ztvm_free(self._h, dptr))
+
+    def upload(self, dptr, array, offset=0):
+        import numpy as np
+        a = np.ascontiguousarray(array)
+        self._chk(self._L.ztvm_upload(self._h, dptr, offset, a.ctypes.data_as(C.c_void_p), a.nbytes))
+
+    def download(self, dptr, nbytes, dtype, offset=0):
+        import numpy as np
+        out = np.empty(nbytes // np.dtype(dtype).itemsize, dtype)
+        self._chk(self._L.ztvm_download(self._h, out.ctypes.data_as(C.c_void_p), dptr, offset, out.nbytes))
+        return out
+
+    def fill(self, dptr, byte, nbytes, offset=0):
+        self._chk(self._L.ztvm_fill(self._h, dptr, offset, byte, nbytes))
+
+    def sync(self):
+        self._chk(self._L.ztvm_sync(self._h))
+
+    def matmul(self, desc):
+        self._chk(self._L.ztvm_matmul(self._h, C.byref(desc)))
+
+    def dequant(self, desc):
+        self._chk(self._L.ztvm_dequant(self._h, C.byref(desc)))
+
+    def record_begin(self):
+        self._chk(self._L.ztvm_record_begin(self._h))
+
+    def record_end(self):
+        cb = C.c_void_p()
+        self._chk(self._L.ztvm_record_end(self._h, C.byref(cb)))
+        return cb
+
+    def submit(self, cb):
+        self._chk(self._L.ztvm_submit(self._h, cb))
+
+    def cmdbuf_destroy(self, cb):
+        self._L.ztvm_cmdbuf_destroy(cb)
+
+    def event(self):
+        e = C.c_void_p()
+        self._chk(self._L.ztvm_event_create(self._h, C.byref(e)))
+        return e
+
+    def event_record(self, e):
+        self._chk(self._L.ztvm_event_record(self._h, e))
+
+    def event_destroy(self, e):
+        self._L.ztvm_event_destroy(e)
+
+    def elapsed_ms(self, start, stop):
+        ms = C.c_float()
+        self._chk(self._L.ztvm_event_elapsed_ms(self._h, start, stop, C.byref(ms)))
+        return ms.value
+
+    def set_option(self, name, value):
+        self._chk(self._L.ztvm_set_option(self._h, name.encode(), int(value)))
+
+    def get_option(self, name):
+        v = C.c_int()
+        self._chk(self._L.ztvm_get_option(self._h, name.encode(), C.byref(v)))
+        return v.value
