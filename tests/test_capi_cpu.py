@@ -1,0 +1,98 @@
+"""The C-ABI library on a machine without a GPU: it loads, exports every symbol
+declared in include/ztvm.h, validates descriptors by the generator's legality
+rules (src/compiler/shaders/int4_matmul.gen.ts:172-197) and refuses to create a
+context instead of falling back to anything."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "ztvm.h")).read()
+    return sorted(set(re.findall(r"ZTVM_API[^;(]*?\b(ztvm_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(capi):
+    lib = capi.load()
+    names = declared_symbols()
+    assert len(names) >= 25
+    for n in names:
+        assert hasattr(lib, n), n
+    assert sorted(capi.EXPORTS) == names
+    assert lib.ztvm_abi_version() == 1
+
+
+def test_desc_struct_matches_header_layout(capi):
+    d = capi.MatmulDesc
+    assert ctypes.sizeof(d) == 16 * 4 + 6 * 8
+    assert d.out.offset == 64 and d.ids.offset == 64 + 40
+
+
+def good(capi, **kw):
+    base = dict(bits=4, affine=1, out_f32=0, kernel=0, M=1, N=64, k_packed=512, scales_per_row=64,
+                out=0x1000, in_=0x2000, scales=0x3000, weights=0x4000, biases=0x5000)
+    base.update(kw)
+    return capi.MatmulDesc(**base)
+
+
+def test_validator_accepts_reference_shapes(capi):
+    assert capi.validate(good(capi))[0] == 0
+    assert capi.validate(good(capi, affine=0, scales_per_row=128, biases=0))[0] == 0
+    assert capi.validate(good(capi, bits=3, k_packed=384, scales_per_row=64))[0] == 0
+    moe = good(capi, N=512, k_packed=256, scales_per_row=32, slots=8, tokens=16, in_slot_stride=0, out_slot_stride=1024,
+               in_tok_stride=2048, out_tok_stride=8 * 1024, ids_stride=8, ids=0x6000, experts=256)
+    assert capi.validate(moe)[0] == 0
+    assert capi.resolve(moe) == capi.KERNEL_GEMV
+
+
+@pytest.mark.parametrize("kw,needle", [
+    (dict(bits=5), "bits"),
+    (dict(bits=3, affine=0, k_packed=384, scales_per_row=128, biases=0), "q3 requires affine"),
+    (dict(affine=0, scales_per_row=128, biases=0, slots=8, tokens=1, ids=0x6000, ids_stride=8), "moe requires affine"),
+    (dict(k_packed=0), "K_PACKED"),
+    (dict(k_packed=4, scales_per_row=1), "group"),          # K=32 is not a multiple of 64
+    (dict(scales_per_row=63), "SCALES_PER_ROW"),
+    (dict(bits=3, k_packed=385, scales_per_row=64), "3-bit"),
+    (dict(N=0), "N"),
+    (dict(M=0), "M"),
+    (dict(biases=0), "binding 5"),
+    (dict(out=0), "binding 0"),
+    (dict(in_=0), "binding 1"),
+    (dict(scales=0), "binding 2"),
+    (dict(weights=0), "binding 3"),
+    (dict(weights=0x4004), "aligned"),
+    (dict(in_=0x2002), "aligned"),
+    (dict(out=0x1001), "misaligned"),
+    (dict(slots=8, tokens=2, ids=0, ids_stride=8, out_slot_stride=64), "binding 6"),
+    (dict(slots=8, tokens=2, ids=0x6000, ids_stride=4, out_slot_stride=64), "IDS_STRIDE"),
+    (dict(slots=8, tokens=2, ids=0x6000, ids_stride=8, M=4, out_slot_stride=64), "M must be 1"),
+    (dict(slots=8, tokens=2, ids=0x6000, ids_stride=8, in_slot_stride=4, out_slot_stride=64), "multiples of 8"),
+    (dict(slots=8, tokens=2, ids=0x6000, ids_stride=8, out_slot_stride=8), "overlap"),
+    (dict(kernel=9), "kernel"),
+])
+def test_validator_rejects(capi, kw, needle):
+    rc, why = capi.validate(good(capi, **kw))
+    assert rc == capi.E_INVALID and needle.lower() in why.lower(), (rc, why)
+
+
+def test_explicit_kernel_that_cannot_run_is_an_error(capi):
+    """Never a silent substitution (pickChunkGemm, src/zero-tvm/engine-core.ts:220-245)."""
+    moe = good(capi, N=512, k_packed=256, scales_per_row=32, slots=8, tokens=1, out_slot_stride=512, ids_stride=8,
+               ids=0x6000, kernel=capi.KERNEL_GEMM)
+    rc, why = capi.validate(moe)
+    assert rc == capi.E_UNSUPPORTED and "asked for" in why
+    with pytest.raises(capi.ZtvmError):
+        capi.resolve(moe)
+
+
+def test_no_device_is_a_loud_error(capi):
+    import subprocess, sys
+    code = ("import importlib,sys; sys.path.insert(0,%r); c=importlib.import_module('zero-tvm_amd.host.capi');\n"
+            "try:\n  c.Context(0); print('CREATED')\nexcept c.ZtvmError as e:\n  print('ERR', e.code)") % ROOT
+    env = dict(os.environ, HIP_VISIBLE_DEVICES="-1", ROCR_VISIBLE_DEVICES="-1")
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=env, timeout=120).stdout
+    assert "ERR -4" in out, out

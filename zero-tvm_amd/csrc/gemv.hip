@@ -23,8 +23,7 @@
 namespace ztvm {
 namespace {
 
-constexpr int WG_THREADS = 256;
-constexpr int WAVES = WG_THREADS / 64;
+constexpr int MAX_WG_THREADS = 512;
 
 struct GemvParams {
   void* out;
@@ -38,17 +37,23 @@ struct GemvParams {
   uint32_t slots, in_slot_stride, out_slot_stride, in_tok_stride, out_tok_stride, ids_stride, experts;
 };
 
-struct __attribute__((packed, aligned(4))) Words3 {
-  uint32_t a, b, c;
-};
+// Three words of a 3-bit chunk: 12 bytes at a 4-byte aligned address.
+typedef uint32_t words3 __attribute__((ext_vector_type(3), aligned(4)));
 
 // LDS layout of x for chunk c: piece j (8 halves, 16 bytes) sits at 16-byte
 // slot (c/64)*256 + j*64 + c%64, so the 64 lanes of one ds_read_b128 touch 64
 // consecutive slots.
 __device__ __forceinline__ uint32_t x_slot(uint32_t c, uint32_t j) { return (c >> 6) * 256u + j * 64u + (c & 63u); }
 
+// One (tile, pass) worth of global loads for ROWS rows of a wave.
+template <int ROWS>
+struct Frag {
+  uint32_t w[ROWS][4];
+  _Float16 s[ROWS], b[ROWS];
+};
+
 template <int BITS, bool AFFINE, int LPR, int ROWS>
-__global__ __launch_bounds__(WG_THREADS) void gemv_kernel(const GemvParams p) {
+__global__ __launch_bounds__(MAX_WG_THREADS) void gemv_kernel(const GemvParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
   constexpr int SUB = 64 / LPR;          // row slots per wave load
   constexpr int RPW = ROWS * SUB;        // rows per wave step
@@ -57,6 +62,7 @@ __global__ __launch_bounds__(WG_THREADS) void gemv_kernel(const GemvParams p) {
   const uint32_t tid = threadIdx.x;
   const uint32_t lane = tid & 63u;
   const uint32_t wave = tid >> 6;
+  const uint32_t waves = blockDim.x >> 6;
   const uint32_t lk = lane % LPR;
   const uint32_t sub = lane / LPR;
 
@@ -77,128 +83,142 @@ __global__ __launch_bounds__(WG_THREADS) void gemv_kernel(const GemvParams p) {
     out_base = (size_t)token * p.out_tok_stride + (size_t)slot * p.out_slot_stride;
   }
 
+  UnpackConsts kc;
+  kc.init();
+
+  // Loads of one (tile, pass). Rows past N and chunks past K are clamped to a
+  // valid address (their contribution is masked later), so no lane diverges.
+  auto issue = [&](Frag<ROWS>& f, uint32_t tile, uint32_t pass) {
+    const uint32_t c = pass * LPR + lk;
+    const uint32_t cc = c < p.nchunks ? c : p.nchunks - 1;
+    const uint32_t g = AFFINE ? (cc >> 1) : cc;
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+      uint32_t rr = tile * RPW + r * SUB + sub;
+      rr = rr < p.N ? rr : p.N - 1;
+      const uint32_t* wp = wbase + (size_t)rr * p.k_packed + (size_t)cc * WPC;
+      if (BITS == 4) {
+        const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp));
+        f.w[r][0] = v.x; f.w[r][1] = v.y; f.w[r][2] = v.z; f.w[r][3] = v.w;
+      } else {
+        const words3 v = __builtin_nontemporal_load(reinterpret_cast<const words3*>(wp));
+        f.w[r][0] = v.x; f.w[r][1] = v.y; f.w[r][2] = v.z; f.w[r][3] = 0;
+      }
+      f.s[r] = sbase[(size_t)rr * p.spr + g];
+      if (AFFINE) f.b[r] = bbase[(size_t)rr * p.spr + g];
+    }
+  };
+
+  // The wave's first loads go out before anything else, so the weight stream
+  // starts while x is still being staged.
+  const uint32_t wave_stride = gridDim.x * waves;
+  uint32_t tile = blockIdx.x * waves + wave, pass = 0;
+  bool have = tile < p.ntiles;
+  Frag<ROWS> fa, fb;
+  if (have) issue(fa, tile, 0);
+
   // ---- stage x: each thread converts whole chunks -------------------------
   h8* xs_pieces = reinterpret_cast<h8*>(smem);
   const uint32_t padded_chunks = (p.nchunks + 63u) & ~63u;
   float* xsum = reinterpret_cast<float*>(smem + (size_t)padded_chunks * 64u);
-  for (uint32_t c = tid; c < padded_chunks; c += WG_THREADS) {
+  for (uint32_t c = tid; c < p.nchunks; c += blockDim.x) {
     float s = 0.f;
-    if (c < p.nchunks) {
-      const h8* src = reinterpret_cast<const h8*>(x + (size_t)c * 32u);
+    const h8* src = reinterpret_cast<const h8*>(x + (size_t)c * 32u);
 #pragma unroll
-      for (int j = 0; j < 4; j++) {
-        const h8 v = src[j];
-        h8 o;
+    for (int j = 0; j < 4; j++) {
+      const h8 v = src[j];
+      h8 o;
 #pragma unroll
-        for (int sl = 0; sl < 8; sl++) o[sl] = v[value_in_slot(sl)];
-        xs_pieces[x_slot(c, j)] = o;
+      for (int sl = 0; sl < 8; sl++) o[sl] = v[value_in_slot(sl)];
+      xs_pieces[x_slot(c, j)] = o;
 #pragma unroll
-        for (int i = 0; i < 8; i++) s += (float)v[i];
-      }
-    } else {
-      const h8 z = {0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll
-      for (int j = 0; j < 4; j++) xs_pieces[x_slot(c, j)] = z;
+      for (int i = 0; i < 8; i++) s += (float)v[i];
     }
     xsum[c] = s;
   }
   __syncthreads();
 
-  const uint32_t wave_global = blockIdx.x * WAVES + wave;
-  const uint32_t wave_stride = gridDim.x * WAVES;
+  float acc[ROWS];
+#pragma unroll
+  for (int r = 0; r < ROWS; r++) acc[r] = 0.f;
 
-  for (uint32_t tile = wave_global; tile < p.ntiles; tile += wave_stride) {
-    float acc[ROWS];
-    uint32_t row[ROWS];
+  // One pipeline stage: prefetch the next (tile, pass) into `nxt`, then consume `cur`.
+  auto stage = [&](const Frag<ROWS>& cur, Frag<ROWS>& nxt) {
+    uint32_t ntile = tile, npass = pass + 1;
+    if (npass == p.npasses) { npass = 0; ntile += wave_stride; }
+    const bool nhave = ntile < p.ntiles;
+    if (nhave) issue(nxt, ntile, npass);
+    // keep the loads above where they are: the scheduler would otherwise sink
+    // the small scale/bias loads down to their first use
+    __builtin_amdgcn_sched_barrier(0);
+
+    const uint32_t c = pass * LPR + lk;
+    const bool live = c < p.nchunks;
+    const uint32_t cc = live ? c : p.nchunks - 1;
+    h2 xv[16];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const h8 v = xs_pieces[x_slot(cc, j)];
+      xv[4 * j + 0] = (h2){v[0], v[1]};
+      xv[4 * j + 1] = (h2){v[2], v[3]};
+      xv[4 * j + 2] = (h2){v[4], v[5]};
+      xv[4 * j + 3] = (h2){v[6], v[7]};
+    }
+    const float xs = xsum[cc];
 #pragma unroll
     for (int r = 0; r < ROWS; r++) {
-      acc[r] = 0.f;
-      const uint32_t rr = tile * RPW + r * SUB + sub;
-      row[r] = rr < p.N ? rr : p.N - 1;  // clamp loads, mask the store
+      h2 q[16];
+      if (BITS == 4) unpack4_chunk(cur.w[r][0], cur.w[r][1], cur.w[r][2], cur.w[r][3], q, kc);
+      else unpack3_chunk(cur.w[r][0], cur.w[r][1], cur.w[r][2], q, kc);
+      float d0 = 0.f, d1 = 0.f;
+#pragma unroll
+      for (int i = 0; i < 16; i += 2) {
+        d0 = __builtin_amdgcn_fdot2(q[i], xv[i], d0, false);
+        d1 = __builtin_amdgcn_fdot2(q[i + 1], xv[i + 1], d1, false);
+      }
+      const float dot = d0 + d1;
+      const float s = (float)cur.s[r];
+      const float term = AFFINE ? __builtin_fmaf(s, dot, (float)cur.b[r] * xs) : s * __builtin_fmaf(-7.f, xs, dot);
+      acc[r] += live ? term : 0.f;
     }
 
-    for (uint32_t pass = 0; pass < p.npasses; pass++) {
-      const uint32_t c = pass * LPR + lk;
-      const bool live = c < p.nchunks;
-      const uint32_t cc = live ? c : p.nchunks - 1;
-
-      // issue every global load of this pass first
-      uint32_t w[ROWS][4];
-      _Float16 sc[ROWS], bi[ROWS];
+    if (pass == p.npasses - 1) {
 #pragma unroll
       for (int r = 0; r < ROWS; r++) {
-        const uint32_t* wp = wbase + (size_t)row[r] * p.k_packed + (size_t)cc * WPC;
-        if (BITS == 4) {
-          const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp));
-          w[r][0] = v.x; w[r][1] = v.y; w[r][2] = v.z; w[r][3] = v.w;
-        } else {
-          const Words3 v = *reinterpret_cast<const Words3*>(wp);  // 12 bytes, 4-byte aligned
-          w[r][0] = v.a; w[r][1] = v.b; w[r][2] = v.c; w[r][3] = 0;
+        const float total = group_sum_to_last_lane<LPR>(acc[r]);
+        acc[r] = 0.f;
+        const uint32_t rr = tile * RPW + r * SUB + sub;
+        if (lk == LPR - 1 && rr < p.N) {
+          if (p.out_f32) reinterpret_cast<float*>(p.out)[out_base + rr] = total;
+          else reinterpret_cast<_Float16*>(p.out)[out_base + rr] = (_Float16)total;
         }
-        const uint32_t g = AFFINE ? (cc >> 1) : cc;
-        sc[r] = sbase[(size_t)row[r] * p.spr + g];
-        if (AFFINE) bi[r] = bbase[(size_t)row[r] * p.spr + g];
-      }
-      // keep the compiler from sinking the small scale/bias loads down to their
-      // first use, where their latency would be exposed once per pass
-      __builtin_amdgcn_sched_barrier(0);
-
-      h2 xv[16];
-#pragma unroll
-      for (int j = 0; j < 4; j++) {
-        const h8 v = xs_pieces[x_slot(cc, j)];
-        xv[4 * j + 0] = (h2){v[0], v[1]};
-        xv[4 * j + 1] = (h2){v[2], v[3]};
-        xv[4 * j + 2] = (h2){v[4], v[5]};
-        xv[4 * j + 3] = (h2){v[6], v[7]};
-      }
-      const float xs = xsum[cc];
-
-#pragma unroll
-      for (int r = 0; r < ROWS; r++) {
-        h2 q[16];
-        if (BITS == 4) unpack4_chunk(w[r][0], w[r][1], w[r][2], w[r][3], q);
-        else unpack3_chunk(w[r][0], w[r][1], w[r][2], q);
-        float d0 = 0.f, d1 = 0.f;
-#pragma unroll
-        for (int i = 0; i < 16; i += 2) {
-          d0 = __builtin_amdgcn_fdot2(q[i], xv[i], d0, false);
-          d1 = __builtin_amdgcn_fdot2(q[i + 1], xv[i + 1], d1, false);
-        }
-        const float dot = d0 + d1;
-        const float s = (float)sc[r];
-        const float term = AFFINE ? s * dot + (float)bi[r] * xs : s * (dot - 7.f * xs);
-        acc[r] += live ? term : 0.f;
       }
     }
+    tile = ntile; pass = npass; have = nhave;
+  };
 
-#pragma unroll
-    for (int r = 0; r < ROWS; r++) {
-      const float total = group_sum_to_last_lane<LPR>(acc[r]);
-      const uint32_t rr = tile * RPW + r * SUB + sub;
-      if (lk == LPR - 1 && rr < p.N) {
-        if (p.out_f32) reinterpret_cast<float*>(p.out)[out_base + rr] = total;
-        else reinterpret_cast<_Float16*>(p.out)[out_base + rr] = (_Float16)total;
-      }
-    }
+  while (have) {
+    stage(fa, fb);
+    if (!have) break;
+    stage(fb, fa);
   }
 }
 
 template <int BITS, bool AFFINE, int LPR, int ROWS>
-hipError_t launch_one(const GemvParams& p, dim3 grid, size_t smem, hipStream_t s) {
-  hipLaunchKernelGGL((gemv_kernel<BITS, AFFINE, LPR, ROWS>), grid, dim3(WG_THREADS), smem, s, p);
+hipError_t launch_one(const GemvParams& p, dim3 grid, uint32_t threads, size_t smem, hipStream_t s) {
+  hipLaunchKernelGGL((gemv_kernel<BITS, AFFINE, LPR, ROWS>), grid, dim3(threads), smem, s, p);
   return hipGetLastError();
 }
 
 template <int BITS, bool AFFINE>
-hipError_t launch_fmt(const GemvParams& p, int lpr, int rows, dim3 grid, size_t smem, hipStream_t s) {
+hipError_t launch_fmt(const GemvParams& p, int lpr, int rows, dim3 grid, uint32_t threads, size_t smem, hipStream_t s) {
   if (lpr == 64) {
-    if (rows == 4) return launch_one<BITS, AFFINE, 64, 4>(p, grid, smem, s);
-    if (rows == 2) return launch_one<BITS, AFFINE, 64, 2>(p, grid, smem, s);
-    return launch_one<BITS, AFFINE, 64, 1>(p, grid, smem, s);
+    if (rows == 4) return launch_one<BITS, AFFINE, 64, 4>(p, grid, threads, smem, s);
+    if (rows == 2) return launch_one<BITS, AFFINE, 64, 2>(p, grid, threads, smem, s);
+    return launch_one<BITS, AFFINE, 64, 1>(p, grid, threads, smem, s);
   }
-  if (lpr == 32) return launch_one<BITS, AFFINE, 32, 2>(p, grid, smem, s);
-  return launch_one<BITS, AFFINE, 16, 2>(p, grid, smem, s);
+  if (lpr == 32) return launch_one<BITS, AFFINE, 32, 2>(p, grid, threads, smem, s);
+  return launch_one<BITS, AFFINE, 16, 2>(p, grid, threads, smem, s);
 }
 
 }  // namespace
@@ -219,31 +239,32 @@ hipError_t launch_gemv(const MatmulArgs& a, const Tune& t, hipStream_t s) {
   p.npasses = (p.nchunks + lpr - 1) / lpr;
   const uint32_t pairs = p.moe ? a.slots * a.tokens : 1;
 
-  int rows = 2;
-  if (lpr == 64) {
-    rows = t.gemv_rows ? t.gemv_rows : (p.npasses >= 4 ? 2 : 4);
-    // few rows: prefer more, smaller tiles so every CU gets work
-    while (rows > 1 && (uint64_t)((a.N + rows - 1) / rows) * pairs < (uint64_t)t.num_cus * WAVES * 2) rows >>= 1;
-  }
+  // Launch shape (measured on MI355X): one row per wave step and 8-wave
+  // workgroups, 3 per CU, stream best for wide rows; narrow rows (several rows
+  // per wave load) use 2 steps in flight.
+  const int cus = t.num_cus;
+  int rows = lpr == 64 ? (t.gemv_rows ? t.gemv_rows : 1) : 2;
+  const uint32_t waves = t.gemv_waves ? t.gemv_waves : 8;
+  uint32_t gx = (uint32_t)cus * (t.gemv_wg_per_cu ? t.gemv_wg_per_cu : 3);
   const uint32_t rpw = rows * (64 / lpr);
   p.ntiles = (a.N + rpw - 1) / rpw;
 
   const uint32_t padded_chunks = (p.nchunks + 63u) & ~63u;
   const size_t smem = (size_t)padded_chunks * 64 + (size_t)padded_chunks * 4;
 
-  const uint32_t wg_tiles = (p.ntiles + WAVES - 1) / WAVES;
-  const int wg_per_cu = t.gemv_wg_per_cu ? t.gemv_wg_per_cu : 4;
-  uint32_t gx = (uint32_t)t.num_cus * wg_per_cu / (pairs < 1 ? 1 : pairs);
+  const uint32_t wg_tiles = (p.ntiles + waves - 1) / waves;
+  gx = gx / pairs;
   if (gx < 1) gx = 1;
   if (gx > wg_tiles) gx = wg_tiles;
   const dim3 grid(gx, pairs, 1);
+  const uint32_t threads = waves * 64;
 
   // dense M>1 handled by the caller looping rows; here one activation row
   if (a.bits == 4) {
-    if (a.affine) return launch_fmt<4, true>(p, lpr, rows, grid, smem, s);
-    return launch_fmt<4, false>(p, lpr, rows, grid, smem, s);
+    if (a.affine) return launch_fmt<4, true>(p, lpr, rows, grid, threads, smem, s);
+    return launch_fmt<4, false>(p, lpr, rows, grid, threads, smem, s);
   }
-  return launch_fmt<3, true>(p, lpr, rows, grid, smem, s);
+  return launch_fmt<3, true>(p, lpr, rows, grid, threads, smem, s);
 }
 
 }  // namespace ztvm

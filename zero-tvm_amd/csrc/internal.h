@@ -24,6 +24,7 @@ struct Tune {
   int num_cus = 256;
   int gemv_wg_per_cu = 0;   // workgroups resident per CU for the streaming GEMV
   int gemv_rows = 0;        // rows per wave step (1, 2 or 4)
+  int gemv_waves = 0;       // waves per workgroup (4..8)
   int skinny_wg_per_cu = 0;
   int gemm_tile = 0;        // 0 auto
   int gemm_xcd_swizzle = 1;

@@ -33,47 +33,69 @@ __host__ __device__ constexpr int slot_of(int i) { return (i & 3) * 2 + (i >> 2)
 // Inverse: which value sits in slot s.
 __host__ __device__ constexpr int value_in_slot(int s) { return (s >> 1) + (s & 1) * 4; }
 
+// (a & mask) | c in ONE instruction. A VOP3 instruction of this ISA may read a
+// single scalar operand, so the OR constant is kept in a vector register
+// (callers hoist it out of their loops); left to itself the compiler emits a
+// separate AND and OR, each with its own literal.
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t c_vgpr) {
+  uint32_t d;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "s"(mask), "v"(c_vgpr));
+  return d;
+}
+
+// OR constants of the unpackers, materialised once per kernel in VGPRs.
+struct UnpackConsts {
+  uint32_t c4_lo, c4_hi;  // 4-bit: 1024|1024 and 64|64
+  uint32_t c3_a, c3_b;    // 3-bit: 64|1024 and 8|128
+  __device__ __forceinline__ void init() {
+    asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(c4_lo));
+    asm volatile("v_mov_b32 %0, 0x54005400" : "=v"(c4_hi));
+    asm volatile("v_mov_b32 %0, 0x64005400" : "=v"(c3_a));
+    asm volatile("v_mov_b32 %0, 0x58004800" : "=v"(c3_b));
+  }
+};
+
 // One u32 of eight 4-bit values (value i at bits [4i,4i+4)) -> 4 x h2 holding
 // the exact integers 0..15 in slot order.
-__device__ __forceinline__ void unpack4_block(uint32_t w, h2 q[4]) {
+__device__ __forceinline__ void unpack4_block(uint32_t w, h2 q[4], const UnpackConsts& k) {
   const h2 k1024 = {(_Float16)1024.f, (_Float16)1024.f};
   const h2 k64 = {(_Float16)64.f, (_Float16)64.f};
   const uint32_t w8 = w >> 8;
-  q[0] = as_h2((w & 0x000F000Fu) | 0x64006400u) - k1024;   // v0, v4
-  q[1] = as_h2((w & 0x00F000F0u) | 0x54005400u) - k64;     // v1, v5
-  q[2] = as_h2((w8 & 0x000F000Fu) | 0x64006400u) - k1024;  // v2, v6
-  q[3] = as_h2((w8 & 0x00F000F0u) | 0x54005400u) - k64;    // v3, v7
+  q[0] = as_h2(and_or(w, 0x000F000Fu, k.c4_lo)) - k1024;   // v0, v4
+  q[1] = as_h2(and_or(w, 0x00F000F0u, k.c4_hi)) - k64;     // v1, v5
+  q[2] = as_h2(and_or(w8, 0x000F000Fu, k.c4_lo)) - k1024;  // v2, v6
+  q[3] = as_h2(and_or(w8, 0x00F000F0u, k.c4_hi)) - k64;    // v3, v7
 }
 
 // Two pre-shifted views of a 24-bit window of eight 3-bit values:
 //   lo_view = window << 4  (v0 at bit 4, v1 at bit 7, v4 at bit 16, v5 at bit 19)
 //   hi_view = window >> 2  (v2 at bit 4, v3 at bit 7, v6 at bit 16, v7 at bit 19)
 // Bits outside the four fields may hold anything.
-__device__ __forceinline__ void unpack3_views(uint32_t lo_view, uint32_t hi_view, h2 q[4]) {
+__device__ __forceinline__ void unpack3_views(uint32_t lo_view, uint32_t hi_view, h2 q[4], const UnpackConsts& k) {
   const h2 ka = {(_Float16)64.f, (_Float16)1024.f};  // fields at r=4 (lo half) and r=0 (hi half)
   const h2 kb = {(_Float16)8.f, (_Float16)128.f};    // fields at r=7 (lo half) and r=3 (hi half)
-  q[0] = as_h2((lo_view & 0x00070070u) | 0x64005400u) - ka;  // v0, v4
-  q[1] = as_h2((lo_view & 0x00380380u) | 0x58004800u) - kb;  // v1, v5
-  q[2] = as_h2((hi_view & 0x00070070u) | 0x64005400u) - ka;  // v2, v6
-  q[3] = as_h2((hi_view & 0x00380380u) | 0x58004800u) - kb;  // v3, v7
+  q[0] = as_h2(and_or(lo_view, 0x00070070u, k.c3_a)) - ka;  // v0, v4
+  q[1] = as_h2(and_or(lo_view, 0x00380380u, k.c3_b)) - kb;  // v1, v5
+  q[2] = as_h2(and_or(hi_view, 0x00070070u, k.c3_a)) - ka;  // v2, v6
+  q[3] = as_h2(and_or(hi_view, 0x00380380u, k.c3_b)) - kb;  // v3, v7
 }
 
 // 32 consecutive 3-bit values = 96 bits = three words (the row bitstream is
 // LSB-first and 32-value chunks are word aligned). Block b is the 24-bit
 // window at stream bit 24b; the views are taken straight from the stream with
 // funnel shifts. q[4*b + j] is pair j of block b.
-__device__ __forceinline__ void unpack3_chunk(uint32_t w0, uint32_t w1, uint32_t w2, h2 q[16]) {
-  unpack3_views(w0 << 4, w0 >> 2, q + 0);                                                        // bits  0..23
-  unpack3_views(__builtin_amdgcn_alignbit(w1, w0, 20), __builtin_amdgcn_alignbit(w1, w0, 26), q + 4);   // bits 24..47
-  unpack3_views(__builtin_amdgcn_alignbit(w2, w1, 12), __builtin_amdgcn_alignbit(w2, w1, 18), q + 8);   // bits 48..71
-  unpack3_views(w2 >> 4, w2 >> 10, q + 12);                                                      // bits 72..95
+__device__ __forceinline__ void unpack3_chunk(uint32_t w0, uint32_t w1, uint32_t w2, h2 q[16], const UnpackConsts& k) {
+  unpack3_views(w0 << 4, w0 >> 2, q + 0, k);                                                        // bits  0..23
+  unpack3_views(__builtin_amdgcn_alignbit(w1, w0, 20), __builtin_amdgcn_alignbit(w1, w0, 26), q + 4, k);   // bits 24..47
+  unpack3_views(__builtin_amdgcn_alignbit(w2, w1, 12), __builtin_amdgcn_alignbit(w2, w1, 18), q + 8, k);   // bits 48..71
+  unpack3_views(w2 >> 4, w2 >> 10, q + 12, k);                                                      // bits 72..95
 }
 
-__device__ __forceinline__ void unpack4_chunk(uint32_t w0, uint32_t w1, uint32_t w2, uint32_t w3, h2 q[16]) {
-  unpack4_block(w0, q + 0);
-  unpack4_block(w1, q + 4);
-  unpack4_block(w2, q + 8);
-  unpack4_block(w3, q + 12);
+__device__ __forceinline__ void unpack4_chunk(uint32_t w0, uint32_t w1, uint32_t w2, uint32_t w3, h2 q[16], const UnpackConsts& k) {
+  unpack4_block(w0, q + 0, k);
+  unpack4_block(w1, q + 4, k);
+  unpack4_block(w2, q + 8, k);
+  unpack4_block(w3, q + 12, k);
 }
 
 // Sum over all 64 lanes (LANES=64), or over each aligned group of LANES lanes,

@@ -153,6 +153,7 @@ const Option kOptions[] = {
     {"num_cus", &Tune::num_cus},
     {"gemv.wg_per_cu", &Tune::gemv_wg_per_cu},
     {"gemv.rows", &Tune::gemv_rows},
+    {"gemv.waves", &Tune::gemv_waves},
     {"skinny.wg_per_cu", &Tune::skinny_wg_per_cu},
     {"gemm.tile", &Tune::gemm_tile},
     {"gemm.xcd_swizzle", &Tune::gemm_xcd_swizzle},
