@@ -17,6 +17,8 @@ struct ztvm_ctx {
   hipStream_t stream = nullptr;
   bool recording = false;
   Tune tune;
+  void* scratch = nullptr;  // group sums of the activations for the GEMM's bias term
+  size_t scratch_bytes = 0;
   std::string err;
   hipDeviceProp_t prop;
 };
@@ -184,6 +186,8 @@ int ztvm_create(int device, ztvm_ctx** out) {
   }
   HIP_TRY(nullptr, hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
   c->tune.num_cus = c->prop.multiProcessorCount > 0 ? c->prop.multiProcessorCount : 256;
+  c->scratch_bytes = 4u << 20;
+  HIP_TRY(nullptr, hipMalloc(&c->scratch, c->scratch_bytes));
   *out = c;
   return ZTVM_OK;
 }
@@ -195,6 +199,7 @@ void ztvm_destroy(ztvm_ctx* ctx) {
     (void)hipStreamSynchronize(ctx->stream);
     (void)hipStreamDestroy(ctx->stream);
   }
+  if (ctx->scratch) (void)hipFree(ctx->scratch);
   delete ctx;
 }
 
@@ -286,7 +291,22 @@ int ztvm_matmul(ztvm_ctx* ctx, const ztvm_matmul_desc* desc) {
   if (fam < 0) return fail(ctx, fam, "ztvm_matmul: %s", why);
   switch (fam) {
     case ZTVM_KERNEL_SKINNY: HIP_TRY(ctx, launch_skinny(a, ctx->tune, ctx->stream)); break;
-    case ZTVM_KERNEL_GEMM: HIP_TRY(ctx, launch_gemm(a, ctx->tune, ctx->stream)); break;
+    case ZTVM_KERNEL_GEMM: {
+      const size_t need = gemm_scratch_bytes(a);
+      if (need > ctx->scratch_bytes) {
+        // growing means a free + malloc, which a command buffer cannot hold
+        if (ctx->recording)
+          return fail(ctx, ZTVM_E_UNSUPPORTED, "ztvm_matmul: this GEMM needs %zu bytes of scratch (have %zu); dispatch it once outside a recording first", need, ctx->scratch_bytes);
+        HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+        HIP_TRY(ctx, hipFree(ctx->scratch));
+        ctx->scratch = nullptr;
+        ctx->scratch_bytes = 0;
+        HIP_TRY(ctx, hipMalloc(&ctx->scratch, need));
+        ctx->scratch_bytes = need;
+      }
+      HIP_TRY(ctx, launch_gemm(a, ctx->tune, ctx->scratch, ctx->stream));
+      break;
+    }
     default: {
       // one streaming pass per activation row
       const uint32_t M = a.slots ? 1 : a.M;
