@@ -60,8 +60,9 @@ def test_symmetric_g32(ctx, capi, synth, oracle, K, N, out_f32):
         y = ctx.download(out, N * esz, np.float32 if out_f32 else np.float16).astype(np.float64)
     ref = oracle.gemm(oracle.MODE_FORMULA_F32, 4, False, 1, N, K, x, w, s, None, threads=8)[0]
     assert rel_err(y, ref, 1e-2) < 1e-2
-    if out_f32:  # LM-head logits keep f32 precision
-        assert rel_err(y, ref, 1e-2) < 1e-4
+    if out_f32:  # LM-head logits keep f32 precision: error far below an f16 ulp of the typical output
+        ref64 = oracle.gemm(oracle.MODE_FORMULA_F64, 4, False, 1, N, K, x, w, s, None, threads=8)[0]
+        assert rel_err(y, ref64, 1.0) < 1e-5
 
 
 def moe_case(synth, E, N, K, tokens, slots, bits, shared_input):

@@ -69,8 +69,14 @@ __global__ __launch_bounds__(256) void dequant_kernel(const DequantParams p) {
     for (int i = 0; i < 32; i += 8) {
       h8 w;
 #pragma unroll
-      for (int j = 0; j < 8; j++)
-        w[j] = (_Float16)(AFFINE ? __builtin_fmaf((float)q[i + j], s, b) : ((float)q[i + j] - 7.f) * s);
+      for (int j = 0; j < 8; j++) {
+        // The f32 value must exist before it is narrowed: the mixed-precision FMA the
+        // compiler would otherwise pick (f16 result straight from the exact sum)
+        // rounds ONCE, while the format's definition rounds to f32 and then to f16.
+        float v = AFFINE ? __builtin_fmaf((float)q[i + j], s, b) : ((float)q[i + j] - 7.f) * s;
+        asm volatile("" : "+v"(v));
+        w[j] = (_Float16)v;
+      }
       *reinterpret_cast<h8*>(out + i) = w;
     }
   }

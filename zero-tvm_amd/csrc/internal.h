@@ -25,12 +25,17 @@ struct Tune {
   int gemv_wg_per_cu = 0;   // workgroups resident per CU for the streaming GEMV
   int gemv_rows = 0;        // rows per wave step (1, 2 or 4)
   int gemv_waves = 0;       // waves per workgroup (4..8)
+  int gemv_path = 0;        // 0/1: the f16 dot2 kernel; 2: the int8 matrix-core kernel (opt-in)
+  int i8_ksplit = 0;        // waves sharing one tile in the int8 GEMV (1, 2 or 4)
+  int i8_wg_per_cu = 0;
   int skinny_wg_per_cu = 0;
   int gemm_tile = 0;        // 0 auto
   int gemm_xcd_swizzle = 1;
 };
 
 hipError_t launch_gemv(const MatmulArgs& a, const Tune& t, hipStream_t s);
+hipError_t launch_gemv_i8(const MatmulArgs& a, const Tune& t, hipStream_t s);
+bool gemv_i8_supports(const MatmulArgs& a);
 hipError_t launch_skinny(const MatmulArgs& a, const Tune& t, hipStream_t s);
 hipError_t launch_gemm(const MatmulArgs& a, const Tune& t, void* scratch, hipStream_t s);
 size_t gemm_scratch_bytes(const MatmulArgs& a);

@@ -156,6 +156,9 @@ const Option kOptions[] = {
     {"gemv.wg_per_cu", &Tune::gemv_wg_per_cu},
     {"gemv.rows", &Tune::gemv_rows},
     {"gemv.waves", &Tune::gemv_waves},
+    {"gemv.path", &Tune::gemv_path},
+    {"i8.ksplit", &Tune::i8_ksplit},
+    {"i8.wg_per_cu", &Tune::i8_wg_per_cu},
     {"skinny.wg_per_cu", &Tune::skinny_wg_per_cu},
     {"gemm.tile", &Tune::gemm_tile},
     {"gemm.xcd_swizzle", &Tune::gemm_xcd_swizzle},
@@ -308,15 +311,27 @@ int ztvm_matmul(ztvm_ctx* ctx, const ztvm_matmul_desc* desc) {
       break;
     }
     default: {
-      // one streaming pass per activation row
+      // streaming passes over the weights: up to four activation rows per pass on
+      // the int8 matrix-core kernel, one row per pass on the f16 dot2 kernel
       const uint32_t M = a.slots ? 1 : a.M;
       const size_t out_elt = a.out_f32 ? 4 : 2;
-      for (uint32_t m = 0; m < M; m++) {
+      uint32_t m = 0;
+      while (m < M) {
         MatmulArgs r = a;
-        r.M = 1;
         r.in = a.in + (size_t)m * a.K;
         r.out = reinterpret_cast<char*>(a.out) + (size_t)m * a.N * out_elt;
-        HIP_TRY(ctx, launch_gemv(r, ctx->tune, ctx->stream));
+        r.M = a.slots ? 1 : (M - m < 4 ? M - m : 4);
+        const bool i8 = ctx->tune.gemv_path == 2 && gemv_i8_supports(r);
+        if (ctx->tune.gemv_path == 2 && !i8)
+          return fail(ctx, ZTVM_E_UNSUPPORTED, "ztvm_matmul: gemv.path=2 asks for the int8 kernel, which cannot run this dispatch (bits=%u, K=%u)", a.bits, a.K);
+        if (i8) {
+          HIP_TRY(ctx, launch_gemv_i8(r, ctx->tune, ctx->stream));
+          m += r.M;
+        } else {
+          r.M = 1;
+          HIP_TRY(ctx, launch_gemv(r, ctx->tune, ctx->stream));
+          m += 1;
+        }
       }
     }
   }
