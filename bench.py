@@ -23,6 +23,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+# HBM bytes per GEMV launch (mean of the three configs[1] shapes) from two `rocprofv3 --pmc` runs of
+# `bench.py --pmc` (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from a 256 MiB copy);
+# summary in profiles/gemv_int4_configs1_hbm_traffic.md
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 26.96e6
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense f16 MFMA, published
 
 GEMV_SHAPES = [("ffn_gate_or_up", 4096, 14336), ("ffn_down", 14336, 4096), ("qkv_fused", 4096, 6144)]
@@ -122,6 +126,9 @@ def main():
     ap.add_argument("--sets", type=int, default=8, help="distinct weight sets rotated through (8 x 80 MB > 256 MB cache)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the per-shape, GEMM, MoE and int3 extras")
+    ap.add_argument("--pmc", action="store_true",
+                    help="counter-collection mode for `rocprofv3 --pmc`: a few eager launches of a 256 MiB copy "
+                         "(calibration) and of each configs[1] GEMV, no timing")
     ap.add_argument("--option", action="append", default=[], help="name=value launch knob (ztvm_set_option)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -138,6 +145,21 @@ def main():
         k, v = opt.split("=")
         ctx.set_option(k, int(v))
     info = ctx.device_info()
+
+    if args.pmc:
+        nbytes = 256 << 20
+        src, dst = ctx.alloc(nbytes), ctx.alloc(nbytes)
+        ctx.fill(src, 1, nbytes)
+        for _ in range(3):
+            ctx.copy(dst, src, nbytes)
+        for i, (_, K, N) in enumerate(GEMV_SHAPES):
+            descs = [make_desc(capi, 4, K, N, 1, upload_set(ctx, synth, K, N, 4, salt=r)[0]) for r in range(4)]
+            for r in range(8):
+                ctx.matmul(descs[r % 4])
+        ctx.sync()
+        ctx.close()
+        print(json.dumps({"pmc_mode": True, "copy_bytes": nbytes}))
+        return
 
     # ---- headline: rotating weight sets, three GEMVs per step ------------------
     sets = []
@@ -174,7 +196,7 @@ def main():
                                "per step, %d rotating weight sets" % args.sets,
                    "device": info["name"], "compute_units": info["compute_units"]},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": GEMV_TRAFFIC_BYTES_PER_LAUNCH,
                      "kernel": "ztvm::gemv_kernel<4,true,64,*>", "bytes_per_launch": step_bytes / 3.0,
                      "avg_launch_us": round(avg_launch_us, 3), "launches": launches},
     }
@@ -188,6 +210,27 @@ def main():
             wb = synth.weight_bytes(N, K)
             extra["gemv_%s_K%d_N%d" % (name, K, N)] = {"us": round(ms * 1e3, 3), "GB/s": round(wb / ms / 1e6, 1),
                                                        "hbm_frac": round(wb / ms / 1e6 / HBM_PEAK_GBS, 4)}
+        # prefill GEMM (configs[2]): K=4096, N=14336, M in {128, 512, 2048}
+        gsets = []
+        for r in range(3):
+            bufs, host = upload_set(ctx, synth, 4096, 14336, 4, salt=100 + r, M=2048)
+            gsets.append((bufs, host))
+        for M in (128, 512, 2048):
+            descs = [make_desc(capi, 4, 4096, 14336, M, b, kernel=capi.KERNEL_GEMM) for b, _ in gsets]
+            verify(ctx, oracle, capi, descs[0], gsets[0][1], 4, 4096, 14336, M)
+            reps = 12 if M <= 512 else 4
+            ms = timed_graph(ctx, [lambda d=descs[j % 3]: ctx.matmul(d) for j in range(reps * 3)]) / (reps * 3)
+            tf = 2.0 * M * 4096 * 14336 / ms / 1e9
+            extra["gemm_M%d_K4096_N14336" % M] = {"us": round(ms * 1e3, 2), "TFLOP/s": round(tf, 1),
+                                                  "mfma_f16_frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
+        # int3 decode GEMV (configs[4], M=1)
+        i3 = [upload_set(ctx, synth, 4096, 14336, 3, salt=200 + r) for r in range(8)]
+        d3 = [make_desc(capi, 3, 4096, 14336, 1, b) for b, _ in i3]
+        verify(ctx, oracle, capi, d3[0], i3[0][1], 3, 4096, 14336, 1)
+        ms = timed_graph(ctx, [lambda d=d3[j % 8]: ctx.matmul(d) for j in range(160)]) / 160
+        wb = synth.weight_bytes(14336, 4096, bits=3)
+        extra["gemv_int3_K4096_N14336"] = {"us": round(ms * 1e3, 3), "GB/s": round(wb / ms / 1e6, 1),
+                                           "hbm_frac": round(wb / ms / 1e6 / HBM_PEAK_GBS, 4)}
         result["extra"] = extra
 
     if not args.no_cpu:

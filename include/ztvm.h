@@ -132,6 +132,9 @@ ZTVM_API int ztvm_upload(ztvm_ctx* ctx, uint64_t dst, size_t dst_off, const void
 ZTVM_API int ztvm_download(ztvm_ctx* ctx, void* dst, uint64_t src, size_t src_off, size_t bytes);
 /* Fill with a repeated byte, ordered on the stream (a kernel, so it may be recorded). */
 ZTVM_API int ztvm_fill(ztvm_ctx* ctx, uint64_t dst, size_t dst_off, int byte, size_t bytes);
+/* copyBufferToBuffer (tests/kernels/gpu.mjs:107-110): device-to-device, ordered on the stream (a kernel,
+ * so it may be recorded). Both addresses and the size must be multiples of 16 bytes. */
+ZTVM_API int ztvm_copy(ztvm_ctx* ctx, uint64_t dst, uint64_t src, size_t bytes);
 ZTVM_API int ztvm_sync(ztvm_ctx* ctx);
 
 /* ---- dispatch ----------------------------------------------------------- */

@@ -93,7 +93,20 @@ __global__ __launch_bounds__(256) void fill16_kernel(u32x4* dst, uint32_t word, 
   for (size_t i = (size_t)blockIdx.x * 256u + threadIdx.x; i < n16; i += stride) dst[i] = v;
 }
 
+__global__ __launch_bounds__(256) void copy16_kernel(u32x4* __restrict__ dst, const u32x4* __restrict__ src, size_t n16) {
+  const size_t stride = (size_t)gridDim.x * 256u;
+  for (size_t i = (size_t)blockIdx.x * 256u + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
+}
+
 }  // namespace
+
+hipError_t launch_copy(void* dst, const void* src, size_t bytes, hipStream_t s) {
+  const size_t n16 = bytes / 16;
+  size_t blocks = (n16 + 255) / 256;
+  if (blocks > 8192) blocks = 8192;
+  hipLaunchKernelGGL(copy16_kernel, dim3((uint32_t)blocks), dim3(256), 0, s, reinterpret_cast<u32x4*>(dst), reinterpret_cast<const u32x4*>(src), n16);
+  return hipGetLastError();
+}
 
 hipError_t launch_dequant(const MatmulArgs& a, hipStream_t s) {
   DequantParams p{};

@@ -344,7 +344,7 @@ hipError_t launch_gemm(const MatmulArgs& a, const Tune& t, void* scratch, hipStr
     hipLaunchKernelGGL(xsum_kernel, dim3((n + 255) / 256), dim3(256), 0, s, a.in, reinterpret_cast<_Float16*>(scratch), a.M, a.K, a.spr);
   }
   int tile = t.gemm_tile;
-  if (!tile) tile = a.M > 128 ? 2 : 1;
+  if (!tile) tile = a.M > 256 ? 3 : (a.M > 64 ? 2 : 1);  // measured: 256x128 wins from M=512 up
   switch (tile) {
     case 3: return launch_tile<4, 2>(p, a.affine, s);  // 256 x 128, 8 waves
     case 2: return launch_tile<2, 2>(p, a.affine, s);  // 128 x 128, 4 waves

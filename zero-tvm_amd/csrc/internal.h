@@ -40,6 +40,7 @@ hipError_t launch_skinny(const MatmulArgs& a, const Tune& t, hipStream_t s);
 hipError_t launch_gemm(const MatmulArgs& a, const Tune& t, void* scratch, hipStream_t s);
 size_t gemm_scratch_bytes(const MatmulArgs& a);
 hipError_t launch_dequant(const MatmulArgs& a, hipStream_t s);
+hipError_t launch_copy(void* dst, const void* src, size_t bytes, hipStream_t s);
 hipError_t launch_fill(void* dst, int byte, size_t bytes, hipStream_t s);
 
 bool skinny_supports(const MatmulArgs& a);

@@ -258,6 +258,14 @@ int ztvm_fill(ztvm_ctx* ctx, uint64_t dst, size_t off, int byte, size_t bytes) {
   return ZTVM_OK;
 }
 
+int ztvm_copy(ztvm_ctx* ctx, uint64_t dst, uint64_t src, size_t bytes) {
+  if (!ctx || !dst || !src) return fail(ctx, ZTVM_E_INVALID, "ztvm_copy: null argument");
+  if ((dst | src | bytes) & 15u) return fail(ctx, ZTVM_E_INVALID, "ztvm_copy: addresses and size must be multiples of 16 bytes");
+  if (!bytes) return ZTVM_OK;
+  HIP_TRY(ctx, launch_copy(reinterpret_cast<void*>(dst), reinterpret_cast<const void*>(src), bytes, ctx->stream));
+  return ZTVM_OK;
+}
+
 int ztvm_sync(ztvm_ctx* ctx) {
   if (!ctx) return fail(nullptr, ZTVM_E_INVALID, "null context");
   if (ctx->recording) return fail(ctx, ZTVM_E_INVALID, "ztvm_sync while recording a command buffer");

@@ -15,7 +15,7 @@ E_INVALID, E_HIP, E_UNSUPPORTED, E_NODEVICE = -1, -2, -3, -4
 
 EXPORTS = [
     "ztvm_abi_version", "ztvm_last_error", "ztvm_create", "ztvm_destroy", "ztvm_device_info",
-    "ztvm_alloc", "ztvm_free", "ztvm_upload", "ztvm_download", "ztvm_fill", "ztvm_sync",
+    "ztvm_alloc", "ztvm_free", "ztvm_upload", "ztvm_download", "ztvm_fill", "ztvm_copy", "ztvm_sync",
     "ztvm_matmul_validate", "ztvm_matmul_resolve", "ztvm_matmul", "ztvm_dequant",
     "ztvm_record_begin", "ztvm_record_end", "ztvm_submit", "ztvm_cmdbuf_destroy",
     "ztvm_event_create", "ztvm_event_destroy", "ztvm_event_record", "ztvm_event_elapsed_ms",
@@ -60,6 +60,7 @@ def load():
     L.ztvm_upload.argtypes = [vp, C.c_uint64, C.c_size_t, vp, C.c_size_t]
     L.ztvm_download.argtypes = [vp, vp, C.c_uint64, C.c_size_t, C.c_size_t]
     L.ztvm_fill.argtypes = [vp, C.c_uint64, C.c_size_t, C.c_int, C.c_size_t]
+    L.ztvm_copy.argtypes = [vp, C.c_uint64, C.c_uint64, C.c_size_t]
     L.ztvm_sync.argtypes = [vp]
     L.ztvm_matmul_validate.argtypes = [C.POINTER(MatmulDesc), C.c_char_p, C.c_size_t]
     L.ztvm_matmul_resolve.argtypes = [C.POINTER(MatmulDesc)]
@@ -148,6 +149,9 @@ class Context:
 
     def fill(self, dptr, byte, nbytes, offset=0):
         self._chk(self._L.ztvm_fill(self._h, dptr, offset, byte, nbytes))
+
+    def copy(self, dst, src, nbytes):
+        self._chk(self._L.ztvm_copy(self._h, dst, src, nbytes))
 
     def sync(self):
         self._chk(self._L.ztvm_sync(self._h))
