@@ -1,0 +1,56 @@
+// Typings of the JavaScript host layer (index.js) for TypeScript callers such as the reference engine.
+export interface Int4MatmulOpts {
+  outF32?: boolean; rowsPerWG?: 1 | 4 | 8; subgroups?: boolean; m?: 1 | 4; vec4?: boolean; vec4Half?: boolean
+  mDyn?: boolean; affine?: boolean; moe?: boolean; q3?: boolean
+}
+export interface Pipeline {
+  readonly label: string; readonly affine: boolean; readonly bits: 3 | 4; readonly outF32: boolean
+  readonly moe: boolean; readonly runtimeM: boolean; readonly fixedM: number; readonly kernel: number
+}
+export interface MatmulDesc {
+  bits: number; affine: number; out_f32: number; kernel: number; M: number; N: number; k_packed: number; scales_per_row: number
+  slots?: number; tokens?: number; in_slot_stride?: number; out_slot_stride?: number; in_tok_stride?: number
+  out_tok_stride?: number; ids_stride?: number; experts?: number
+  out: bigint; in: bigint; scales: bigint; weights: bigint; biases?: bigint; ids?: bigint
+}
+export declare class Uniform { words: number[]; writeU32(byteOffset: number, value: number): void }
+export interface ZtvmBuffer { readonly size: number; readonly label: string; readonly addr: bigint; destroy(): void }
+export type BindEntry = ZtvmBuffer | { buffer: ZtvmBuffer; offset: number; size: number } | Uniform
+export interface BindGroup { pipeline: Pipeline; pod: Uniform }
+export declare class Device {
+  constructor(index?: number)
+  close(): void
+  info(): { name: string; computeUnits: number; hbmBytes: bigint }
+  createBuffer(size: number, label?: string): ZtvmBuffer
+  writeBuffer(buf: ZtvmBuffer, offset: number, data: ArrayBufferView | ArrayBuffer): void
+  readBuffer(buf: ZtvmBuffer, offset?: number, bytes?: number): ArrayBuffer
+  fill(buf: ZtvmBuffer, byte: number): void
+  uniformBuf(data: number[]): Uniform
+  createPipeline(entry: string): Pipeline
+  bg(pipeline: Pipeline, bufs: BindEntry[]): BindGroup
+  descriptor(group: BindGroup, wgX?: number, wgY?: number, wgZ?: number): MatmulDesc
+  dispatch(pipeline: Pipeline, group: BindGroup, wgX: number, wgY?: number, wgZ?: number): void
+  beginEncoder(): void
+  finishEncoder(): unknown
+  submit(cmdbuf: unknown): void
+  sync(): void
+}
+export declare const KERNEL: { AUTO: 0; GEMV: 1; SKINNY: 2; GEMM: 3 }
+export declare const INT4_MATMUL_VARIANTS: ReadonlyArray<Int4MatmulOpts>
+export declare const GEMM_ENTRIES: ReadonlyArray<string>
+export declare const ALL_ENTRIES: ReadonlyArray<string>
+export declare function int4MatmulEntry(opts?: Int4MatmulOpts): string
+export declare function checkOpts(opts?: Int4MatmulOpts): void
+export declare function createPipeline(entry: string): Pipeline
+export declare function resolveMatmul(variant: string, available: Set<string> | string[], vec4?: boolean, k?: number,
+  vec4Half?: boolean, affine?: boolean, vec4Affine?: boolean): { pipeline: string; pipelineF32: string; rowsPerWG: number; label: string }
+export declare function resolveChunkCap(opts: { chunkCap?: number }, spec: { maxChunkCap?: number }, sgmatAvail: boolean): number
+export type ChunkGemmName = 'e5' | 'sgmat' | 'tiled' | 'matvec'
+export declare function pickChunkGemm(caps: { want?: ChunkGemmName; chunkTiled: boolean; dimsOK: boolean; capTiles64: boolean
+  e5Ready: boolean; sgmatReady: boolean; cap: number }): { used: ChunkGemmName; rejected: string | null }
+export declare function foldGridX(total: number, maxX?: number): { x: number; z: number }
+export declare function densePod(K: number, N: number, bits?: number, affine?: boolean, M?: number): number[]
+export declare function moePods(dModel: number, ffn: number, slots: number, bits?: number): { gate: number[]; down: number[] }
+export declare function validate(desc: MatmulDesc): { code: number; why: string }
+export declare function resolve(desc: MatmulDesc): number
+export declare function abiVersion(): number
