@@ -24,13 +24,21 @@
 //   workgroup  WM x WN waves, each wave a 64 x 64 output tile (2 x 2 blocks of
 //              v_mfma_f32_32x32x16_f16); A operand = activations, B operand =
 //              weights, so lanes of D run along n and stores are contiguous
-//   K step     64 = one affine group (two symmetric groups), double-buffered LDS
-//   LDS rows   64 f16 = eight 16-byte chunks, chunk index XOR (row & 7): the
-//              lanes served together by a 128-bit read hit distinct banks
+//   K step     64 = one affine group (two symmetric groups), three LDS stages
+//   LDS rows   64 f16 = eight 16-byte chunks, chunk index XOR bits 1..3 of the
+//              row: the 16 lanes served together by a 128-bit read cover all
+//              64 banks (measured 560 B/ns per CU, same as a linear read)
+//   pipeline   step s multiplies stage s%3; the activations of step s+2 go
+//              global -> LDS without passing registers, the packed weights of
+//              step s+2 are unpacked from registers into the same stage, the
+//              fragments of step s+1 are read while those of step s retire,
+//              and the previous run's partial sums are folded between MFMAs;
+//              one barrier per step
 //   grid       one workgroup per tile, ids remapped so that the tiles sharing
 //              a weight panel run on the same XCD (same L2)
 #include "internal.h"
 #include "quant.h"
+#include <utility>
 
 namespace ztvm {
 namespace {
@@ -44,11 +52,15 @@ struct GemmParams {
   const _Float16* scales;
   const uint32_t* weights;
   const _Float16* biases;
-  const _Float16* xs16;  // [M][2*G]: hi halves then lo halves of the group sums
+  const _Float16* xs16;  // [M][xs_stride]: hi halves, lo halves of the group sums, zero padding
   uint32_t M, N, K, k_packed, spr;
-  uint32_t mtiles, ntiles, nsteps, bias_steps;
+  uint32_t mtiles, ntiles, nsteps, bias_steps, xs_stride;
   uint32_t xcd_swizzle;
 };
+
+// LDS swizzle: a 128-bit read serves 16 lanes per cycle = two 128-byte rows of banks, and rows of
+// equal parity share a bank half, so the chunk index is XOR-ed with bits 1..3 of the row.
+__device__ __forceinline__ uint32_t swz(uint32_t row) { return (row >> 1) & 7u; }
 
 // One packed word -> eight exact f16 integers in natural k order. A byte holds
 // values (2j, 2j+1); replicating the low byte pair into both halves of a word
@@ -66,12 +78,20 @@ __device__ __forceinline__ h8 unpack_word_natural(uint32_t w, uint32_t c_mixed) 
   return (h8){p0.x, p0.y, p1.x, p1.y, p2.x, p2.y, p3.x, p3.y};
 }
 
-// Group sums of the activations: xs16[m][g] = f16(xs), xs16[m][G+g] = f16(xs - hi).
+// Group sums of the activations, one row of XS_STRIDE f16 per activation row:
+// xs16[m][g] = f16(xs), xs16[m][G+g] = f16(xs - hi), zero from 2G up to the stride.
 __global__ __launch_bounds__(256) void xsum_kernel(const _Float16* __restrict__ in, _Float16* __restrict__ xs16, uint32_t M,
-                                                  uint32_t K, uint32_t G) {
+                                                  uint32_t K, uint32_t G, uint32_t xs_stride) {
   const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
-  if (idx >= M * G) return;
-  const uint32_t m = idx / G, g = idx % G;
+  const uint32_t half = xs_stride / 2;  // columns handled per row: g < half covers [0,G) plus its share of the padding
+  if (idx >= M * half) return;
+  const uint32_t m = idx / half, g = idx % half;
+  _Float16* row = xs16 + (size_t)m * xs_stride;
+  if (g >= G) {  // padding columns 2G + 2(g-G), +1
+    row[2 * G + 2 * (g - G)] = (_Float16)0.f;
+    row[2 * G + 2 * (g - G) + 1] = (_Float16)0.f;
+    return;
+  }
   const h8* src = reinterpret_cast<const h8*>(in + (size_t)m * K + (size_t)g * 64);
   float s = 0.f;
 #pragma unroll
@@ -82,27 +102,56 @@ __global__ __launch_bounds__(256) void xsum_kernel(const _Float16* __restrict__ 
   }
   const _Float16 hi = (_Float16)s;
   const _Float16 lo = (_Float16)(s - (float)hi);
-  xs16[(size_t)m * 2 * G + g] = hi;
-  xs16[(size_t)m * 2 * G + G + g] = lo;
+  row[g] = hi;
+  row[G + g] = lo;
 }
+
+typedef const __attribute__((address_space(1))) void* gptr_t;
+typedef __attribute__((address_space(3))) void* lptr_t;
+
+template <int... Is, class F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, Is...>, F&& f) {
+  (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(std::make_integer_sequence<int, N>{}, f);
+}
+
+constexpr int NSTAGE = 3;
+
+// The 16 MFMAs of a step as 8 pairs (block row i, k slice ks) x 2 block columns. A run of pairs
+// accumulates one group into one partial set (set = i); affine: 64-k groups, runs of 4 pairs;
+// symmetric: 32-k groups, runs of 2 pairs.
+template <bool AFFINE>
+struct Seq {
+  static constexpr int RUN = AFFINE ? 4 : 2;
+  static constexpr int I(int p) { return AFFINE ? p / 4 : (p / 2) % 2; }
+  static constexpr int KSL(int p) { return AFFINE ? p % 4 : (p / 4) * 2 + p % 2; }
+  static constexpr int GRP(int p) { return AFFINE ? 0 : p / 4; }
+};
 
 template <int WM, int WN, bool AFFINE>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) {
-  constexpr int THREADS = 64 * WM * WN;
+  using S = Seq<AFFINE>;
+  constexpr int WAVES = WM * WN, THREADS = 64 * WAVES;
   constexpr int TM = 64 * WM, TN = 64 * WN;
-  constexpr int A_LOADS = TM * CHUNKS / THREADS;  // 16-byte loads per thread per step
+  constexpr int A_LOADS = TM * CHUNKS / THREADS;  // 16-byte direct-to-LDS loads per lane per step
   constexpr int W_WORDS = TN * 8 / THREADS;       // packed words per thread per step
   static_assert(A_LOADS >= 1 && (W_WORDS == 2 || W_WORDS == 4 || W_WORDS == 8), "tile/thread mismatch");
   constexpr int W_TPR = 8 / W_WORDS;              // threads per weight row
   constexpr int SCALES = AFFINE ? 1 : 2;          // groups per step
   constexpr int SC_LOADS = (TN * SCALES + THREADS - 1) / THREADS;
+  constexpr uint32_t ROW_BYTES = CHUNKS * 16;
+  constexpr uint32_t STAGE_BYTES = (TM + TN) * ROW_BYTES;
+  constexpr uint32_t W_BASE = TM * ROW_BYTES;          // weight rows follow the activation rows of a stage
+  constexpr uint32_t SC_BASE = NSTAGE * STAGE_BYTES;   // float [NSTAGE][TN][SCALES]
+  constexpr uint32_t SC_STAGE = TN * SCALES * 4;
 
   extern __shared__ __align__(16) unsigned char smem[];
-  constexpr int STAGE_CHUNKS = (TM + TN) * CHUNKS;
-  h8* lds = reinterpret_cast<h8*>(smem);                                         // [2][STAGE_CHUNKS]
-  float* lds_s = reinterpret_cast<float*>(smem + 2 * STAGE_CHUNKS * 16);         // [2][TN][SCALES]
 
-  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const uint32_t tid = threadIdx.x, lane = tid & 63u;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const uint32_t wm = wave / WN, wn = wave % WN;
 
   // workgroup id -> tile: ids sharing an XCD (id % 8) take consecutive tiles,
@@ -116,114 +165,96 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
   uint32_t c_mixed;  // OR constant: 64 in the high half, 1024 in the low half
   asm volatile("v_mov_b32 %0, 0x54006400" : "=v"(c_mixed));
 
-  u32x4 areg[A_LOADS];
-  uint32_t wreg[W_WORDS];
-  _Float16 sreg[SC_LOADS];
-  const uint32_t total_steps = p.nsteps + p.bias_steps;
-  const uint32_t G = p.spr;
-
-  const uint32_t w_row = tid / W_TPR, w_part = tid % W_TPR;  // this thread's weight row and word group
-  uint32_t w_n = n0 + w_row;
-  w_n = w_n < p.N ? w_n : p.N - 1;  // clamped rows are never stored
-
-  // step < nsteps: activations + packed weights of k = 64*step ..
-  // step >= nsteps (affine only): group sums + biases, 64 columns of [hi | lo] per step
-  auto load_step = [&](uint32_t step) {
-    if (step < p.nsteps) {
-      const uint32_t k0 = step * KS;
+  // ---- activations: global -> LDS without passing registers. One instruction fills 64
+  // consecutive 16-byte LDS slots (8 rows), slot = lane; the lane fetches the chunk that the
+  // swizzle places there. Rows past M repeat row M-1: they are computed and never stored.
+  const _Float16* a_src[A_LOADS];
+  const _Float16* xs_src[A_LOADS];
 #pragma unroll
-      for (int i = 0; i < A_LOADS; i++) {
-        const uint32_t c = tid + i * THREADS, row = c / CHUNKS, ch = c % CHUNKS;
-        const uint32_t m = m0 + row;
-        u32x4 v = {0, 0, 0, 0};
-        if (m < p.M) v = *reinterpret_cast<const u32x4*>(p.in + (size_t)m * p.K + k0 + ch * 8);
-        areg[i] = v;
-      }
-      const uint32_t* wp = p.weights + (size_t)w_n * p.k_packed + (k0 >> 3) + w_part * W_WORDS;
-      if (W_WORDS == 2) {
-        const u32x2 v = *reinterpret_cast<const u32x2*>(wp);
-        wreg[0] = v.x; wreg[1] = v.y;
-      } else {
+  for (int i = 0; i < A_LOADS; i++) {
+    const uint32_t row = (i * WAVES + wave) * 8 + (lane >> 3);
+    const uint32_t ch = (lane & 7u) ^ swz(row);
+    uint32_t m = m0 + row;
+    m = m < p.M ? m : p.M - 1;
+    a_src[i] = p.in + (size_t)m * p.K + ch * 8;
+    xs_src[i] = p.xs16 + (size_t)m * p.xs_stride + ch * 8;
+  }
+  auto load_a = [&](const _Float16** src, uint32_t stage) __attribute__((always_inline)) {
 #pragma unroll
-        for (int q4 = 0; q4 < W_WORDS / 4; q4++) {
-          const u32x4 v = *reinterpret_cast<const u32x4*>(wp + 4 * q4);
-          wreg[4 * q4 + 0] = v.x; wreg[4 * q4 + 1] = v.y; wreg[4 * q4 + 2] = v.z; wreg[4 * q4 + 3] = v.w;
-        }
-      }
-#pragma unroll
-      for (int i = 0; i < SC_LOADS; i++) {
-        const uint32_t idx = tid + i * THREADS;
-        if (idx < TN * SCALES) {
-          uint32_t n = n0 + idx / SCALES;
-          n = n < p.N ? n : p.N - 1;
-          sreg[i] = p.scales[(size_t)n * p.spr + step * SCALES + idx % SCALES];
-        }
-      }
-    } else {
-      const uint32_t c0 = (step - p.nsteps) * KS;  // column of the [hi | lo] matrix
-#pragma unroll
-      for (int i = 0; i < A_LOADS; i++) {
-        const uint32_t c = tid + i * THREADS, row = c / CHUNKS, ch = c % CHUNKS;
-        const uint32_t m = m0 + row, col = c0 + ch * 8;
-        u32x4 v = {0, 0, 0, 0};
-        if (m < p.M && col < 2 * G) {
-          const _Float16* src = p.xs16 + (size_t)m * 2 * G + col;
-          if (G % 4 == 0) {
-            v = *reinterpret_cast<const u32x4*>(src);
-          } else {  // narrow K: rows of the [hi | lo] matrix are not 16-byte multiples
-            h8 t = {0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll
-            for (int e = 0; e < 8; e++)
-              if (col + e < 2 * G) t[e] = src[e];
-            v = __builtin_bit_cast(u32x4, t);
-          }
-        }
-        areg[i] = v;
-      }
-      // biases: column c of the B matrix is b[n][c mod G]; W_WORDS chunks of 8 columns per thread
-#pragma unroll
-      for (int j = 0; j < W_WORDS; j++) wreg[j] = 0;  // unused in this phase
+    for (int i = 0; i < A_LOADS; i++) {
+      __builtin_amdgcn_global_load_lds((gptr_t)src[i], (lptr_t)(smem + stage * STAGE_BYTES + (i * WAVES + wave) * 1024u), 16, 0, 0);
+      src[i] += KS;
     }
   };
 
-  auto store_step = [&](uint32_t step, uint32_t buf) {
-    h8* a_lds = lds + buf * STAGE_CHUNKS;
-    h8* w_lds = a_lds + TM * CHUNKS;
+  // ---- weights: registers, unpack, LDS
+  const uint32_t w_row = tid / W_TPR, w_part = tid % W_TPR;
+  uint32_t w_n = n0 + w_row;
+  w_n = w_n < p.N ? w_n : p.N - 1;  // clamped rows are never stored
+  const uint32_t* w_src = p.weights + (size_t)w_n * p.k_packed + w_part * W_WORDS;
+  uint32_t w_dst[W_WORDS];
 #pragma unroll
-    for (int i = 0; i < A_LOADS; i++) {
-      const uint32_t c = tid + i * THREADS, row = c / CHUNKS, ch = c % CHUNKS;
-      a_lds[row * CHUNKS + (ch ^ (row & 7u))] = __builtin_bit_cast(h8, areg[i]);
-    }
-    if (step < p.nsteps) {
+  for (int j = 0; j < W_WORDS; j++) w_dst[j] = W_BASE + w_row * ROW_BYTES + (((w_part * W_WORDS + j) ^ swz(w_row)) << 4);
+  // scales: thread -> (column, group of the step); surplus threads repeat the last one
+  const _Float16* sc_src[SC_LOADS];
+  uint32_t sc_dst[SC_LOADS];
 #pragma unroll
-      for (int j = 0; j < W_WORDS; j++) {
-        const uint32_t ch = w_part * W_WORDS + j;
-        w_lds[w_row * CHUNKS + (ch ^ (w_row & 7u))] = unpack_word_natural<AFFINE>(wreg[j], c_mixed);
-      }
-#pragma unroll
-      for (int i = 0; i < SC_LOADS; i++) {
-        const uint32_t idx = tid + i * THREADS;
-        if (idx < TN * SCALES) lds_s[buf * TN * SCALES + idx] = (float)sreg[i];
-      }
+  for (int i = 0; i < SC_LOADS; i++) {
+    uint32_t idx = tid + i * THREADS;
+    idx = idx < TN * SCALES ? idx : TN * SCALES - 1;
+    uint32_t n = n0 + idx / SCALES;
+    n = n < p.N ? n : p.N - 1;
+    sc_src[i] = p.scales + (size_t)n * p.spr + idx % SCALES;
+    sc_dst[i] = SC_BASE + idx * 4;
+  }
+
+  struct WRegs {
+    uint32_t w[W_WORDS];
+    _Float16 s[SC_LOADS];
+  };
+  auto load_w = [&](WRegs& r) __attribute__((always_inline)) {
+    if (W_WORDS == 2) {
+      const u32x2 v = *reinterpret_cast<const u32x2*>(w_src);
+      r.w[0] = v.x; r.w[1] = v.y;
     } else {
-      const uint32_t c0 = (step - p.nsteps) * KS;
 #pragma unroll
-      for (int j = 0; j < W_WORDS; j++) {
-        const uint32_t ch = w_part * W_WORDS + j, col = c0 + ch * 8;
-        h8 v = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (col < 2 * G) {
-          const _Float16* brow = p.biases + (size_t)w_n * G;
-          if (G % 8 == 0) {
-            v = *reinterpret_cast<const h8*>(brow + (col % G));
-          } else {
-#pragma unroll
-            for (int e = 0; e < 8; e++)
-              if (col + e < 2 * G) v[e] = brow[(col + e) % G];
-          }
-        }
-        w_lds[w_row * CHUNKS + (ch ^ (w_row & 7u))] = v;
+      for (int q4 = 0; q4 < W_WORDS / 4; q4++) {
+        const u32x4 v = *reinterpret_cast<const u32x4*>(w_src + 4 * q4);
+        r.w[4 * q4 + 0] = v.x; r.w[4 * q4 + 1] = v.y; r.w[4 * q4 + 2] = v.z; r.w[4 * q4 + 3] = v.w;
       }
     }
+#pragma unroll
+    for (int i = 0; i < SC_LOADS; i++) {
+      r.s[i] = *sc_src[i];
+      sc_src[i] += SCALES;
+    }
+    w_src += KS / 8;
+  };
+  auto store_w_words = [&](const WRegs& r, uint32_t stage, int j0, int j1) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = j0; j < j1; j++)
+      *reinterpret_cast<h8*>(smem + stage * STAGE_BYTES + w_dst[j]) = unpack_word_natural<AFFINE>(r.w[j], c_mixed);
+  };
+  auto store_w_scales = [&](const WRegs& r, uint32_t stage) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < SC_LOADS; i++) *reinterpret_cast<float*>(smem + stage * SC_STAGE + sc_dst[i]) = (float)r.s[i];
+  };
+
+  // ---- operand fragments: lane -> row frow of a 32-row block, k slice fk of the 16
+  const uint32_t frow = lane & 31u, fk = lane >> 5;
+  uint32_t a_rd[KS / 16], b_rd[KS / 16];
+#pragma unroll
+  for (int ks = 0; ks < KS / 16; ks++) {
+    const uint32_t x = frow * ROW_BYTES + (((ks * 2 + fk) ^ swz(frow)) << 4);
+    a_rd[ks] = x + wm * 64 * ROW_BYTES;
+    b_rd[ks] = x + W_BASE + wn * 64 * ROW_BYTES;
+  }
+  const uint32_t sc_rd = SC_BASE + (wn * 64 + frow) * SCALES * 4;
+  auto read_a = [&](uint32_t stage, int i, int ks) __attribute__((always_inline)) {
+    return *reinterpret_cast<const h8*>(smem + stage * STAGE_BYTES + a_rd[ks] + i * 32 * ROW_BYTES);
+  };
+  auto read_b = [&](uint32_t stage, int j, int ks) __attribute__((always_inline)) {
+    return *reinterpret_cast<const h8*>(smem + stage * STAGE_BYTES + b_rd[ks] + j * 32 * ROW_BYTES);
   };
 
   f16v tot[2][2];
@@ -233,62 +264,173 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
     for (int j = 0; j < 2; j++)
 #pragma unroll
       for (int e = 0; e < 16; e++) tot[i][j][e] = 0.f;
-
-  load_step(0);
-  store_step(0, 0);
-  __syncthreads();
-
-  const uint32_t frow = lane & 31u, fk = lane >> 5;  // operand row inside a 32-block, which 8 of the 16 k
   const f16v zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 
-  for (uint32_t step = 0; step < total_steps; step++) {
-    const uint32_t buf = step & 1u;
-    if (step + 1 < total_steps) load_step(step + 1);
-
-    const h8* a_lds = lds + buf * STAGE_CHUNKS;
-    const h8* w_lds = a_lds + TM * CHUNKS;
-    const bool main_phase = step < p.nsteps;
-
-    // PH phases of KS/PH k each; each phase ends with one scale-and-fold
-    constexpr int PH = AFFINE ? 1 : 2;
+  // ---- bias term first (affine): tot = [xs_hi | xs_lo] x biases on the matrix cores, 64 columns
+  // per step, stage 0 only, no overlap (two or three short steps).
+  if (AFFINE) {
+    const uint32_t G = p.spr;
+    const _Float16* brow = p.biases + (size_t)w_n * G;
+    for (uint32_t bs = 0; bs < p.bias_steps; bs++) {
+      load_a(xs_src, 0);
 #pragma unroll
-    for (int ph = 0; ph < PH; ph++) {
-      f16v part[2][2];
+      for (int j = 0; j < W_WORDS; j++) {
+        const uint32_t col = bs * KS + (w_part * W_WORDS + j) * 8;  // column c meets b[n][c mod G]; zero past 2G
+        h8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (col < 2 * G) {
+          if (G % 8 == 0) {
+            v = *reinterpret_cast<const h8*>(brow + (col % G));
+          } else {
 #pragma unroll
-      for (int ks = 0; ks < KS / 16 / PH; ks++) {
-        const uint32_t ch = (ph * (KS / 16 / PH) + ks) * 2 + fk;
+            for (int e = 0; e < 8; e++)
+              if (col + e < 2 * G) v[e] = brow[(col + e) % G];
+          }
+        }
+        *reinterpret_cast<h8*>(smem + w_dst[j]) = v;
+      }
+      __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+      __syncthreads();
+#pragma unroll
+      for (int ks = 0; ks < KS / 16; ks++) {
         h8 af[2], bf[2];
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
-          const uint32_t row = wm * 64 + i * 32 + frow;
-          af[i] = a_lds[row * CHUNKS + (ch ^ (row & 7u))];
-        }
+        for (int i = 0; i < 2; i++) af[i] = read_a(0, i, ks);
 #pragma unroll
-        for (int j = 0; j < 2; j++) {
-          const uint32_t row = wn * 64 + j * 32 + frow;
-          bf[j] = w_lds[row * CHUNKS + (ch ^ (row & 7u))];
-        }
+        for (int j = 0; j < 2; j++) bf[j] = read_b(0, j, ks);
 #pragma unroll
         for (int i = 0; i < 2; i++)
 #pragma unroll
-          for (int j = 0; j < 2; j++)
-            part[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], ks == 0 ? zero : part[i][j], 0, 0, 0);
+          for (int j = 0; j < 2; j++) tot[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], tot[i][j], 0, 0, 0);
       }
-      // fold: the lane's column n is fixed per block column j, so one scale per j
-      float sc[2];
-#pragma unroll
-      for (int j = 0; j < 2; j++) sc[j] = main_phase ? lds_s[(buf * TN + wn * 64 + j * 32 + frow) * SCALES + ph] : 1.f;
-#pragma unroll
-      for (int i = 0; i < 2; i++)
-#pragma unroll
-        for (int j = 0; j < 2; j++)
-#pragma unroll
-          for (int e = 0; e < 16; e++) tot[i][j][e] = __builtin_fmaf(sc[j], part[i][j][e], tot[i][j][e]);
+      __syncthreads();
     }
-
-    if (step + 1 < total_steps) store_step(step + 1, buf ^ 1u);
-    __syncthreads();
   }
+
+  // ---- main loop, software pipelined over three LDS stages. Step s multiplies stage s%3 while
+  //   * the activations of step s+2 stream into stage (s+2)%3 (issued at the top of step s),
+  //   * the packed weights of step s+2 (in registers since step s-1) are unpacked into it,
+  //   * the packed weights of step s+3 are fetched into registers,
+  //   * the operand fragments of step s+1 are read from stage (s+1)%3 as those of step s retire,
+  //   * the partial sums of the previous run are folded into the totals between the MFMAs.
+  h8 Bf[2][KS / 16], Aq[4];
+  f16v part[2][2];
+  float sc[SCALES][2], scp[2];  // scales of this step; of the last group of the previous step
+  WRegs wcur, wnext;
+
+  const uint32_t nsteps = p.nsteps;
+  // prologue: stages 0 and 1 complete, weights of step 2 in registers
+  load_a(a_src, 0);
+  load_w(wcur);
+  store_w_words(wcur, 0, 0, W_WORDS);
+  store_w_scales(wcur, 0);
+  if (nsteps > 1) {
+    load_a(a_src, 1);
+    load_w(wcur);
+    store_w_words(wcur, 1, 0, W_WORDS);
+    store_w_scales(wcur, 1);
+  }
+  if (nsteps > 2) load_w(wcur);
+  __builtin_amdgcn_s_waitcnt(0x0070);
+  __syncthreads();
+  static_for<4>([&](auto pc) {
+    constexpr int pp = decltype(pc)::value;
+    Aq[pp] = read_a(0, S::I(pp), S::KSL(pp));
+  });
+#pragma unroll
+  for (int ks = 0; ks < KS / 16; ks++)
+#pragma unroll
+    for (int j = 0; j < 2; j++) Bf[j][ks] = read_b(0, j, ks);
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++) part[i][j] = zero;
+#pragma unroll
+  for (int j = 0; j < 2; j++) {
+    scp[j] = 0.f;
+#pragma unroll
+    for (int g = 0; g < SCALES; g++) sc[g][j] = 0.f;
+  }
+
+  auto step = [&](auto hot_c, uint32_t cur, uint32_t nxt, uint32_t fill, bool fetch_a, bool fetch_w) __attribute__((always_inline)) {
+    constexpr bool HOT = decltype(hot_c)::value;
+    if (HOT || fetch_w) load_w(wnext);
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      scp[j] = sc[SCALES - 1][j];
+#pragma unroll
+      for (int g = 0; g < SCALES; g++)
+        sc[g][j] = *reinterpret_cast<const float*>(smem + cur * SC_STAGE + sc_rd + (j * 32 * SCALES + g) * 4);
+    }
+    static_for<8>([&](auto pc) {
+      constexpr int pp = decltype(pc)::value;
+      constexpr int i = S::I(pp), ks = S::KSL(pp);
+      constexpr bool first = pp % S::RUN == 0;
+#pragma unroll
+      for (int j = 0; j < 2; j++)
+        part[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(Aq[pp % 4], Bf[j][ks], first ? zero : part[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      // the fragment slot just used takes the pair four places on; after block row 1 the
+      // weight fragments of this k slice are done and the next step's replace them
+      if (pp + 4 < 8) Aq[pp % 4] = read_a(cur, S::I(pp + 4), S::KSL(pp + 4));
+      else Aq[pp % 4] = read_a(nxt, S::I(pp - 4), S::KSL(pp - 4));
+      if (i == 1) {
+#pragma unroll
+        for (int j = 0; j < 2; j++) Bf[j][ks] = read_b(nxt, j, ks);
+      }
+      // fold a slice of the run that ended before this one: tot += scale * part
+      {
+        constexpr int prev = (pp - pp % S::RUN + 8 - S::RUN) % 8;      // first pair of the previous run
+        constexpr int fi = S::I(prev), fg = S::GRP(prev);
+        constexpr bool from_last_step = pp < S::RUN;
+        constexpr int per = 32 / S::RUN, lo = (pp % S::RUN) * per;     // 32 FMAs per run of 2 blocks
+#pragma unroll
+        for (int q = lo; q < lo + per; q++) {
+          const int j = q / 16, e = q % 16;
+          const float s = from_last_step ? scp[j] : sc[fg][j];
+          tot[fi][j][e] = __builtin_fmaf(s, part[fi][j][e], tot[fi][j][e]);
+        }
+      }
+      if (HOT || fetch_a) {
+        constexpr int i0 = pp * A_LOADS / 4, i1 = (pp + 1) * A_LOADS / 4;  // spread over the first four pairs
+#pragma unroll
+        for (int ia = i0; ia < i1 && ia < A_LOADS; ia++) {
+          __builtin_amdgcn_global_load_lds((gptr_t)a_src[ia], (lptr_t)(smem + fill * STAGE_BYTES + (ia * WAVES + wave) * 1024u), 16, 0, 0);
+          a_src[ia] += KS;
+        }
+      }
+      if (HOT || fetch_a) {
+        if (pp == 0) store_w_words(wcur, fill, 0, W_WORDS / 2);
+        if (pp == 1) {
+          store_w_words(wcur, fill, W_WORDS / 2, W_WORDS);
+          store_w_scales(wcur, fill);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    wcur = wnext;
+    // everything this wave fetched or wrote has landed; the empty statements keep the compiler
+    // from moving LDS accesses across the barrier
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  };
+
+  using hot_t = std::integral_constant<bool, true>;
+  using cold_t = std::integral_constant<bool, false>;
+  uint32_t s = 0;
+  // hot: steps whose s+3 is still a main step
+  for (; s + 6 <= nsteps; s += 3) {
+    step(hot_t{}, 0, 1, 2, true, true);
+    step(hot_t{}, 1, 2, 0, true, true);
+    step(hot_t{}, 2, 0, 1, true, true);
+  }
+  for (; s < nsteps; s++) step(cold_t{}, s % 3, (s + 1) % 3, (s + 2) % 3, s + 2 < nsteps, s + 3 < nsteps);
+  // the last run of the last step is still unfolded
+#pragma unroll
+  for (int j = 0; j < 2; j++)
+#pragma unroll
+    for (int e = 0; e < 16; e++) tot[1][j][e] = __builtin_fmaf(sc[SCALES - 1][j], part[1][j][e], tot[1][j][e]);
 
   // D layout of a 32x32 block: lane -> column n = lane % 32, register e -> row 8*(e/4) + 4*(lane/32) + e%4
 #pragma unroll
@@ -310,7 +452,7 @@ hipError_t launch_tile(GemmParams p, bool affine, hipStream_t s) {
   p.mtiles = (p.M + TM - 1) / TM;
   p.ntiles = (p.N + TN - 1) / TN;
   const dim3 grid(p.mtiles * p.ntiles);
-  const size_t smem = 2 * (size_t)(TM + TN) * CHUNKS * 16 + 2 * (size_t)TN * 2 * sizeof(float);
+  const size_t smem = NSTAGE * ((size_t)(TM + TN) * CHUNKS * 16 + (size_t)TN * (affine ? 1 : 2) * sizeof(float));
   if (affine) {
     auto k = gemm_kernel<WM, WN, true>;
     if (smem > 64 * 1024) (void)hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
@@ -324,11 +466,12 @@ hipError_t launch_tile(GemmParams p, bool affine, hipStream_t s) {
 }
 
 }  // namespace
-
 // 4-bit, f16 output, dense, K a multiple of 64.
 bool gemm_supports(const MatmulArgs& a) { return a.slots == 0 && a.bits == 4 && !a.out_f32 && a.K % KS == 0; }
 
-size_t gemm_scratch_bytes(const MatmulArgs& a) { return a.affine ? (size_t)a.M * 2 * a.spr * sizeof(_Float16) : 0; }
+static uint32_t xs_stride_of(const MatmulArgs& a) { return (2 * a.spr + KS - 1) / KS * KS; }
+
+size_t gemm_scratch_bytes(const MatmulArgs& a) { return a.affine ? (size_t)a.M * xs_stride_of(a) * sizeof(_Float16) : 0; }
 
 hipError_t launch_gemm(const MatmulArgs& a, const Tune& t, void* scratch, hipStream_t s) {
   GemmParams p{};
@@ -337,11 +480,13 @@ hipError_t launch_gemm(const MatmulArgs& a, const Tune& t, void* scratch, hipStr
   p.xs16 = reinterpret_cast<const _Float16*>(scratch);
   p.M = a.M; p.N = a.N; p.K = a.K; p.k_packed = a.k_packed; p.spr = a.spr;
   p.nsteps = a.K / KS;
-  p.bias_steps = a.affine ? (2 * a.spr + KS - 1) / KS : 0;
+  p.xs_stride = xs_stride_of(a);
+  p.bias_steps = a.affine ? p.xs_stride / KS : 0;
   p.xcd_swizzle = t.gemm_xcd_swizzle;
   if (a.affine) {
-    const uint32_t n = a.M * a.spr;
-    hipLaunchKernelGGL(xsum_kernel, dim3((n + 255) / 256), dim3(256), 0, s, a.in, reinterpret_cast<_Float16*>(scratch), a.M, a.K, a.spr);
+    const uint32_t n = a.M * (p.xs_stride / 2);
+    hipLaunchKernelGGL(xsum_kernel, dim3((n + 255) / 256), dim3(256), 0, s, a.in, reinterpret_cast<_Float16*>(scratch), a.M, a.K, a.spr,
+                       p.xs_stride);
   }
   int tile = t.gemm_tile;
   if (!tile) tile = a.M > 256 ? 3 : (a.M > 64 ? 2 : 1);  // measured: 256x128 wins from M=512 up
