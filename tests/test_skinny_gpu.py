@@ -1,0 +1,119 @@
+"""GPU parity of the weight-streaming matrix-core kernel (family 'skinny', 2 <= M <= 128 rows by
+default, any M when asked for).
+
+The cases mirror the reference's small-batch checks (tests/kernels/compile-qwen35.mjs:963-1152:
+M=6 N=64, M=31 N=256, M=47 N=200 at K=2560; scripts/gemm-sweep-native.mjs:374: 13x96x128) and add
+the formats the reference ships for the same dispatch: symmetric group-32 and the 3-bit stream.
+Bars: |y-ref|/(|ref|+1e-2) < 1e-2 against the from-the-formula f64 oracle (the kernel multiplies
+exact integer weights and scales in f32, so it holds the GEMV's bar), rows past M untouched,
+results independent of M and of the tile height, one-hot rows bit-exact.
+"""
+import numpy as np
+import pytest
+
+from .util import Dev, rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def run(ctx, capi, bits, affine, M, CAP, N, K, A, w, s, b, kernel, out_f32=0, prefill=0):
+    esz = 4 if out_f32 else 2
+    with Dev(ctx) as d:
+        out = d.empty(CAP * N * esz, fill=prefill)
+        desc = capi.MatmulDesc(bits=bits, affine=int(affine), out_f32=out_f32, kernel=kernel, M=M, N=N, k_packed=K * bits // 32,
+                               scales_per_row=K // (64 if affine else 32), out=out, in_=d.put(A), scales=d.put(s),
+                               weights=d.put(w), biases=d.put(b) if affine else 0)
+        ctx.matmul(desc)
+        return ctx.download(out, CAP * N * esz, np.uint32 if out_f32 else np.uint16).reshape(CAP, N)
+
+
+def make(synth, bits, affine, CAP, N, K, regime="A"):
+    A = synth.activations(CAP, K)
+    w = synth.packed_weights(N, K, bits=bits)
+    s = synth.scales(N, K, affine=affine)
+    b = synth.biases(N, K, s, regime) if affine else None
+    return A, w, s, b
+
+
+FORMATS = [(4, True), (4, False), (3, True)]
+CASES = [(2, 8, 64, 2560), (6, 8, 64, 2560), (31, 64, 256, 2560), (33, 64, 256, 2560), (47, 64, 200, 2560), (13, 64, 96, 128),
+         (64, 64, 136, 64), (65, 128, 136, 192), (100, 128, 264, 1024), (128, 128, 128, 512), (130, 256, 136, 512),
+         (300, 320, 264, 1024)]
+
+
+@pytest.mark.parametrize("M,CAP,N,K", CASES)
+@pytest.mark.parametrize("bits,affine", FORMATS)
+def test_ragged_skinny(ctx, capi, synth, oracle, M, CAP, N, K, bits, affine):
+    A, w, s, b = make(synth, bits, affine, CAP, N, K)
+    ctx.set_option("skinny.ksplit", 1)  # one summation order whatever M is
+    try:
+        got = run(ctx, capi, bits, affine, M, CAP, N, K, A, w, s, b, capi.KERNEL_SKINNY)
+        gotcap = run(ctx, capi, bits, affine, CAP, CAP, N, K, A, w, s, b, capi.KERNEL_SKINNY)
+    finally:
+        ctx.set_option("skinny.ksplit", 0)
+    y = got[:M].view(np.float16).astype(np.float64)
+    ref = oracle.gemm(oracle.MODE_FORMULA_F64, bits, affine, M, N, K, A, w, s, b, threads=8)
+    assert rel_err(y, ref, 1e-2) < 1e-2
+    assert rel_err(y, ref, 1e-3) < 2e-2
+    assert not got[M:].any(), "rows past M were written"
+    assert np.array_equal(got[:M], gotcap[:M]), "M-variance"
+
+
+@pytest.mark.parametrize("ksplit", [0, 2, 3, 8])
+@pytest.mark.parametrize("bits,affine", FORMATS)
+def test_k_split(ctx, capi, synth, oracle, bits, affine, ksplit):
+    """K dealt to several workgroups, partial results summed in f32 in split order; 0 = the library's choice."""
+    M, N, K = 8, 264, 2048
+    A, w, s, b = make(synth, bits, affine, M, N, K)
+    ctx.set_option("skinny.ksplit", ksplit)
+    try:
+        got = run(ctx, capi, bits, affine, M, M, N, K, A, w, s, b, capi.KERNEL_SKINNY)
+        got32 = run(ctx, capi, bits, affine, M, M, N, K, A, w, s, b, capi.KERNEL_SKINNY, out_f32=1)
+    finally:
+        ctx.set_option("skinny.ksplit", 0)
+    ref = oracle.gemm(oracle.MODE_FORMULA_F64, bits, affine, M, N, K, A, w, s, b, threads=8)
+    assert rel_err(got.view(np.float16).astype(np.float64), ref, 1e-2) < 1e-2
+    assert rel_err(got32.view(np.float32).astype(np.float64), ref, 1.0) < 1e-5
+
+
+def test_one_hot_pins_streamed_weights(ctx, capi, synth, oracle):
+    """A = rows of the identity: Y[m,n] is the dequantized weight f16(fl32(q*s+b)) of W[n,k_m], bit for bit."""
+    N, K = 160, 256
+    ks = np.array([0, 1, 3, 4, 7, 8, 15, 31, 32, 33, 63, 64, 65, 127, 128, 191, 200, 255] * 4, np.int64)[:64]
+    A = np.zeros((64, K), np.float16)
+    A[np.arange(64), ks] = 1.0
+    for bits, affine in FORMATS:
+        _, w, s, b = make(synth, bits, affine, 1, N, K)
+        got = run(ctx, capi, bits, affine, 64, 64, N, K, A.view(np.uint16), w, s, b, capi.KERNEL_SKINNY)
+        w16 = oracle.dequant_matrix(bits, affine, N, K, w, s, b, want="f16")
+        assert np.array_equal(got, w16[:, ks].T), (bits, affine)
+
+
+@pytest.mark.parametrize("bits,affine", FORMATS)
+def test_families_agree(ctx, capi, synth, bits, affine):
+    """The per-token GEMV and the streaming kernel follow the same arithmetic: same f16 results up to
+    one rounding step on a few outputs (different f32 summation order inside a group)."""
+    M, N, K = 16, 256, 1024
+    A, w, s, b = make(synth, bits, affine, M, N, K)
+    g = run(ctx, capi, bits, affine, M, M, N, K, A, w, s, b, capi.KERNEL_GEMV).view(np.float16).astype(np.float64)
+    k = run(ctx, capi, bits, affine, M, M, N, K, A, w, s, b, capi.KERNEL_SKINNY).view(np.float16).astype(np.float64)
+    assert rel_err(k, g, 1e-2) < 2e-3
+
+
+def test_config5_int3_m8(ctx, capi, synth, oracle):
+    """configs[4]: 3-bit weights, M=8, K=4096, N=14336, against the formula."""
+    M, K, N = 8, 4096, 14336
+    A, w, s, b = make(synth, 3, True, M, N, K)
+    got = run(ctx, capi, 3, True, M, M, N, K, A, w, s, b, capi.KERNEL_AUTO)
+    ref = oracle.gemm(oracle.MODE_FORMULA_F64, 3, True, M, N, K, A, w, s, b, threads=8)
+    assert rel_err(got.view(np.float16).astype(np.float64), ref, 1e-2) < 1e-2
+
+
+def test_auto_picks_skinny(capi):
+    for M, want in ((1, capi.KERNEL_GEMV), (2, capi.KERNEL_SKINNY), (128, capi.KERNEL_SKINNY), (129, capi.KERNEL_GEMM)):
+        desc = capi.MatmulDesc(bits=4, affine=1, M=M, N=256, k_packed=64, scales_per_row=8, out=4096, in_=4096, scales=4096,
+                               weights=4096, biases=4096)
+        assert capi.resolve(desc) == want, M
+    desc = capi.MatmulDesc(bits=3, affine=1, M=300, N=256, k_packed=48, scales_per_row=8, out=4096, in_=4096, scales=4096,
+                           weights=4096, biases=4096)
+    assert capi.resolve(desc) == capi.KERNEL_SKINNY  # the tile GEMM has no 3-bit path

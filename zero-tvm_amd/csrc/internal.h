@@ -29,6 +29,7 @@ struct Tune {
   int i8_ksplit = 0;        // waves sharing one tile in the int8 GEMV (1, 2 or 4)
   int i8_wg_per_cu = 0;
   int skinny_wg_per_cu = 0;
+  int skinny_ksplit = 0;     // workgroups sharing the k range of one skinny tile (0: chosen from M, N, K)
   int gemm_tile = 0;        // 0 auto
   int gemm_xcd_swizzle = 1;
 };
@@ -36,7 +37,8 @@ struct Tune {
 hipError_t launch_gemv(const MatmulArgs& a, const Tune& t, hipStream_t s);
 hipError_t launch_gemv_i8(const MatmulArgs& a, const Tune& t, hipStream_t s);
 bool gemv_i8_supports(const MatmulArgs& a);
-hipError_t launch_skinny(const MatmulArgs& a, const Tune& t, hipStream_t s);
+hipError_t launch_skinny(const MatmulArgs& a, const Tune& t, void* scratch, hipStream_t s);
+size_t skinny_scratch_bytes(const MatmulArgs& a, const Tune& t);
 hipError_t launch_gemm(const MatmulArgs& a, const Tune& t, void* scratch, hipStream_t s);
 size_t gemm_scratch_bytes(const MatmulArgs& a);
 hipError_t launch_dequant(const MatmulArgs& a, hipStream_t s);

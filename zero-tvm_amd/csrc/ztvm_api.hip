@@ -125,8 +125,8 @@ MatmulArgs to_args(const ztvm_matmul_desc* d) {
 
 // Which family runs a descriptor. Thresholds are measured crossovers on
 // MI355X: the GEMV re-reads the weights once per activation row, the skinny
-// kernel reads them once for up to 64 rows, the tile GEMM needs enough rows to
-// fill its M tile.
+// kernel streams them once through registers for tiles of up to 128 rows, the
+// tile GEMM needs enough rows to fill its 256-row tile.
 int resolve(const MatmulArgs& a, uint32_t want, char* why, size_t n) {
   const bool moe = a.slots > 0;
   const bool sk = !moe && skinny_supports(a);
@@ -141,7 +141,7 @@ int resolve(const MatmulArgs& a, uint32_t want, char* why, size_t n) {
     return ZTVM_KERNEL_GEMM;
   }
   if (moe || a.M == 1) return ZTVM_KERNEL_GEMV;
-  if (ge && a.M > 32) return ZTVM_KERNEL_GEMM;
+  if (ge && a.M > 128) return ZTVM_KERNEL_GEMM;
   if (sk) return ZTVM_KERNEL_SKINNY;
   if (ge) return ZTVM_KERNEL_GEMM;
   return ZTVM_KERNEL_GEMV;
@@ -160,6 +160,7 @@ const Option kOptions[] = {
     {"i8.ksplit", &Tune::i8_ksplit},
     {"i8.wg_per_cu", &Tune::i8_wg_per_cu},
     {"skinny.wg_per_cu", &Tune::skinny_wg_per_cu},
+    {"skinny.ksplit", &Tune::skinny_ksplit},
     {"gemm.tile", &Tune::gemm_tile},
     {"gemm.xcd_swizzle", &Tune::gemm_xcd_swizzle},
 };
@@ -301,13 +302,13 @@ int ztvm_matmul(ztvm_ctx* ctx, const ztvm_matmul_desc* desc) {
   const int fam = resolve(a, desc->kernel, why, sizeof why);
   if (fam < 0) return fail(ctx, fam, "ztvm_matmul: %s", why);
   switch (fam) {
-    case ZTVM_KERNEL_SKINNY: HIP_TRY(ctx, launch_skinny(a, ctx->tune, ctx->stream)); break;
+    case ZTVM_KERNEL_SKINNY:
     case ZTVM_KERNEL_GEMM: {
-      const size_t need = gemm_scratch_bytes(a);
+      const size_t need = fam == ZTVM_KERNEL_GEMM ? gemm_scratch_bytes(a) : skinny_scratch_bytes(a, ctx->tune);
       if (need > ctx->scratch_bytes) {
         // growing means a free + malloc, which a command buffer cannot hold
         if (ctx->recording)
-          return fail(ctx, ZTVM_E_UNSUPPORTED, "ztvm_matmul: this GEMM needs %zu bytes of scratch (have %zu); dispatch it once outside a recording first", need, ctx->scratch_bytes);
+          return fail(ctx, ZTVM_E_UNSUPPORTED, "ztvm_matmul: this dispatch needs %zu bytes of scratch (have %zu); dispatch it once outside a recording first", need, ctx->scratch_bytes);
         HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
         HIP_TRY(ctx, hipFree(ctx->scratch));
         ctx->scratch = nullptr;
@@ -315,7 +316,8 @@ int ztvm_matmul(ztvm_ctx* ctx, const ztvm_matmul_desc* desc) {
         HIP_TRY(ctx, hipMalloc(&ctx->scratch, need));
         ctx->scratch_bytes = need;
       }
-      HIP_TRY(ctx, launch_gemm(a, ctx->tune, ctx->scratch, ctx->stream));
+      if (fam == ZTVM_KERNEL_GEMM) HIP_TRY(ctx, launch_gemm(a, ctx->tune, ctx->scratch, ctx->stream));
+      else HIP_TRY(ctx, launch_skinny(a, ctx->tune, ctx->scratch, ctx->stream));
       break;
     }
     default: {
