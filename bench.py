@@ -51,6 +51,12 @@ def upload_set(ctx, synth, K, N, bits, salt, M=1):
     return bufs, (x, w, s, b)
 
 
+def _put(ctx, arr):
+    addr = ctx.alloc(arr.nbytes)
+    ctx.upload(addr, arr)
+    return addr
+
+
 def timed_graph(ctx, launches, reps=1):
     """Record `launches` (callables) into one command buffer, replay once untimed, then time `reps` replays."""
     ctx.record_begin()
@@ -231,6 +237,50 @@ def main():
         wb = synth.weight_bytes(14336, 4096, bits=3)
         extra["gemv_int3_K4096_N14336"] = {"us": round(ms * 1e3, 3), "GB/s": round(wb / ms / 1e6, 1),
                                            "hbm_frac": round(wb / ms / 1e6 / HBM_PEAK_GBS, 4)}
+        # small batches through the weight-streaming kernel: int4 M in {8, 32, 128} and configs[4]'s int3 M=8
+        for bits, M in ((4, 8), (4, 32), (4, 128), (3, 8)):
+            src = gsets if bits == 4 else None
+            if bits == 4:
+                descs = [make_desc(capi, 4, 4096, 14336, M, b) for b, _ in gsets]
+                host0 = gsets[0][1]
+            else:
+                i3m = [upload_set(ctx, synth, 4096, 14336, 3, salt=300 + r, M=M) for r in range(3)]
+                descs = [make_desc(capi, 3, 4096, 14336, M, b) for b, _ in i3m]
+                host0 = i3m[0][1]
+            verify(ctx, oracle, capi, descs[0], host0, bits, 4096, 14336, M)
+            ms = timed_graph(ctx, [lambda d=descs[j % 3]: ctx.matmul(d) for j in range(36)]) / 36
+            wb = synth.weight_bytes(14336, 4096, bits=bits)
+            extra["skinny_int%d_M%d_K4096_N14336" % (bits, M)] = {
+                "us": round(ms * 1e3, 2), "TFLOP/s": round(2.0 * M * 4096 * 14336 / ms / 1e9, 1),
+                "weights_GB/s": round(wb / ms / 1e6, 1), "family": capi.KERNEL_NAMES[capi.resolve(descs[0])]}
+        # MoE expert block (configs[3]): 256 experts, top-8, hidden 2048, intermediate 512; gate + up + down per token batch
+        E, slots, d_model, ffn = 256, 8, 2048, 512
+        moe_w = {}
+        for name, N_, K_ in (("gate", ffn, d_model), ("up", ffn, d_model), ("down", d_model, ffn)):
+            w = synth.packed_weights(N_, K_, experts=E, salt=len(name))
+            sc = synth.scales(N_, K_, experts=E, salt=len(name))
+            bi = synth.biases(N_, K_, sc, experts=E, salt=len(name))
+            moe_w[name] = tuple(_put(ctx, a) for a in (w, sc, bi))
+        for tokens in (1, 16):
+            ids = synth.topk_ids(tokens, slots, E, salt=tokens)
+            d_ids = _put(ctx, ids)
+            x = _put(ctx, synth.activations(tokens, d_model, salt=5))
+            gu = ctx.alloc(tokens * slots * 2 * ffn * 2)
+            out = ctx.alloc(tokens * slots * d_model * 2)
+            gcommon = dict(bits=4, affine=1, M=1, N=ffn, k_packed=d_model // 8, scales_per_row=d_model // 64, slots=slots,
+                           tokens=tokens, in_slot_stride=0, out_slot_stride=2 * ffn, in_tok_stride=d_model,
+                           out_tok_stride=slots * 2 * ffn, ids_stride=slots, experts=E, in_=x, ids=d_ids)
+            dg = capi.MatmulDesc(out=gu, weights=moe_w["gate"][0], scales=moe_w["gate"][1], biases=moe_w["gate"][2], **gcommon)
+            du = capi.MatmulDesc(out=gu + ffn * 2, weights=moe_w["up"][0], scales=moe_w["up"][1], biases=moe_w["up"][2], **gcommon)
+            dd = capi.MatmulDesc(bits=4, affine=1, M=1, N=d_model, k_packed=ffn // 8, scales_per_row=ffn // 64, slots=slots,
+                                 tokens=tokens, in_slot_stride=2 * ffn, out_slot_stride=d_model, in_tok_stride=slots * 2 * ffn,
+                                 out_tok_stride=slots * d_model, ids_stride=slots, experts=E, out=out, in_=gu, ids=d_ids,
+                                 weights=moe_w["down"][0], scales=moe_w["down"][1], biases=moe_w["down"][2])
+            ms = timed_graph(ctx, [lambda d=d_: ctx.matmul(d) for _ in range(20) for d_ in (dg, du, dd)]) / 20
+            distinct = len(set(int(v) for v in ids.reshape(-1)))
+            per_expert = 2 * synth.weight_bytes(ffn, d_model) + synth.weight_bytes(d_model, ffn)
+            extra["moe_block_tokens%d" % tokens] = {"us": round(ms * 1e3, 2), "pairs": tokens * slots, "distinct_experts": distinct,
+                                                     "expert_GB/s": round(distinct * per_expert / ms / 1e6, 1)}
         result["extra"] = extra
 
     if not args.no_cpu:

@@ -64,7 +64,7 @@ struct I8Params {
 // source k offset of byte j of a 16-byte operand piece (even nibbles of a word, then odd)
 __host__ __device__ constexpr int piece_k(int j) { return (j >> 3) * 8 + ((j >> 2) & 1) + (j & 3) * 2; }
 
-constexpr int BATCH = 8;          // units whose loads travel together (8 KB per wave in flight)
+constexpr int BATCH = 4;          // units whose loads travel together (8 KB per wave in flight)
 constexpr int WAVES = 4;
 constexpr uint32_t ZERO_BYTES = 32;  // LDS bytes [0, 32): zeros every idle lane reads
 
