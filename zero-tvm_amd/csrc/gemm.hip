@@ -78,32 +78,30 @@ __device__ __forceinline__ h8 unpack_word_natural(uint32_t w, uint32_t c_mixed) 
   return (h8){p0.x, p0.y, p1.x, p1.y, p2.x, p2.y, p3.x, p3.y};
 }
 
-// Group sums of the activations, one row of XS_STRIDE f16 per activation row:
+// Group sums of the activations, one row of xs_stride f16 per activation row:
 // xs16[m][g] = f16(xs), xs16[m][G+g] = f16(xs - hi), zero from 2G up to the stride.
+// One thread per 16-byte chunk, eight consecutive lanes = one 64-k group, summed across lanes.
 __global__ __launch_bounds__(256) void xsum_kernel(const _Float16* __restrict__ in, _Float16* __restrict__ xs16, uint32_t M,
                                                   uint32_t K, uint32_t G, uint32_t xs_stride) {
   const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
-  const uint32_t half = xs_stride / 2;  // columns handled per row: g < half covers [0,G) plus its share of the padding
-  if (idx >= M * half) return;
-  const uint32_t m = idx / half, g = idx % half;
-  _Float16* row = xs16 + (size_t)m * xs_stride;
-  if (g >= G) {  // padding columns 2G + 2(g-G), +1
-    row[2 * G + 2 * (g - G)] = (_Float16)0.f;
-    row[2 * G + 2 * (g - G) + 1] = (_Float16)0.f;
-    return;
-  }
-  const h8* src = reinterpret_cast<const h8*>(in + (size_t)m * K + (size_t)g * 64);
+  const uint32_t cpr = K / 8, total = M * cpr;  // chunks per row; K % 64 == 0, so groups never straddle a wave
+  const uint32_t pad = xs_stride - 2 * G;
+  if (idx < M * pad) xs16[(size_t)(idx / pad) * xs_stride + 2 * G + idx % pad] = (_Float16)0.f;
+  if (idx >= total) return;
+  const uint32_t m = idx / cpr, c = idx % cpr;
+  const h8 v = *reinterpret_cast<const h8*>(in + (size_t)m * K + (size_t)c * 8);
   float s = 0.f;
 #pragma unroll
-  for (int j = 0; j < 8; j++) {
-    const h8 v = src[j];
-#pragma unroll
-    for (int i = 0; i < 8; i++) s += (float)v[i];
+  for (int i = 0; i < 8; i++) s += (float)v[i];
+  s += __shfl_xor(s, 1);
+  s += __shfl_xor(s, 2);
+  s += __shfl_xor(s, 4);
+  if ((c & 7u) == 0) {
+    const uint32_t g = c >> 3;
+    const _Float16 hi = (_Float16)s;
+    xs16[(size_t)m * xs_stride + g] = hi;
+    xs16[(size_t)m * xs_stride + G + g] = (_Float16)(s - (float)hi);
   }
-  const _Float16 hi = (_Float16)s;
-  const _Float16 lo = (_Float16)(s - (float)hi);
-  row[g] = hi;
-  row[G + g] = lo;
 }
 
 typedef const __attribute__((address_space(1))) void* gptr_t;
@@ -484,7 +482,8 @@ hipError_t launch_gemm(const MatmulArgs& a, const Tune& t, void* scratch, hipStr
   p.bias_steps = a.affine ? p.xs_stride / KS : 0;
   p.xcd_swizzle = t.gemm_xcd_swizzle;
   if (a.affine) {
-    const uint32_t n = a.M * (p.xs_stride / 2);
+    const uint32_t pad = p.xs_stride - 2 * a.spr, cpr = a.K / 8;
+    const uint32_t n = a.M * (cpr > pad ? cpr : pad);  // one thread per chunk, and enough for the padding columns
     hipLaunchKernelGGL(xsum_kernel, dim3((n + 255) / 256), dim3(256), 0, s, a.in, reinterpret_cast<_Float16*>(scratch), a.M, a.K, a.spr,
                        p.xs_stride);
   }

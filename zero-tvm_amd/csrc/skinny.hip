@@ -48,40 +48,37 @@ struct StreamParams {
 
 // Pre-pass: slot-ordered copy of the activations and, for affine weights, the group sums
 // xs16[m][g] = f16(xs), xs16[m][G+g] = f16(xs - hi), zero from 2G up to the stride.
+// One thread per 16-byte chunk, eight consecutive lanes = one 64-k group, summed across lanes.
 __global__ __launch_bounds__(256) void prep_kernel(const _Float16* __restrict__ in, _Float16* __restrict__ inp,
                                                    _Float16* __restrict__ xs16, uint32_t M, uint32_t K, uint32_t xs_stride,
                                                    uint32_t want_xs) {
-  const uint32_t G = K / 64;
-  const uint32_t per_row = want_xs ? (G > xs_stride / 2 ? G : xs_stride / 2) : G;
   const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
-  if (idx >= M * per_row) return;
-  const uint32_t m = idx / per_row, g = idx % per_row;
-  _Float16* xrow = xs16 + (size_t)m * xs_stride;
-  if (g >= G) {  // padding columns 2G + 2(g-G), +1
-    if (2 * G + 2 * (g - G) + 1 < xs_stride) {
-      xrow[2 * G + 2 * (g - G)] = (_Float16)0.f;
-      xrow[2 * G + 2 * (g - G) + 1] = (_Float16)0.f;
-    }
-    return;
+  const uint32_t cpr = K / 8, total = M * cpr, G = K / 64;
+  if (want_xs) {
+    const uint32_t pad = xs_stride - 2 * G;
+    if (idx < M * pad) xs16[(size_t)(idx / pad) * xs_stride + 2 * G + idx % pad] = (_Float16)0.f;
   }
-  const h8* src = reinterpret_cast<const h8*>(in + (size_t)m * K + (size_t)g * 64);
-  h8* dst = reinterpret_cast<h8*>(inp + (size_t)m * K + (size_t)g * 64);
+  if (idx >= total) return;
+  const uint32_t m = idx / cpr, c = idx % cpr;
+  const h8 v = *reinterpret_cast<const h8*>(in + (size_t)m * K + (size_t)c * 8);
+  h8 w;
   float s = 0.f;
 #pragma unroll
-  for (int j = 0; j < 8; j++) {
-    const h8 v = src[j];
-    h8 w;
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-      s += (float)v[i];
-      w[slot_of(i)] = v[i];
-    }
-    dst[j] = w;
+  for (int i = 0; i < 8; i++) {
+    s += (float)v[i];
+    w[slot_of(i)] = v[i];
   }
+  *reinterpret_cast<h8*>(inp + (size_t)m * K + (size_t)c * 8) = w;
   if (want_xs) {
-    const _Float16 hi = (_Float16)s;
-    xrow[g] = hi;
-    xrow[G + g] = (_Float16)(s - (float)hi);
+    s += __shfl_xor(s, 1);
+    s += __shfl_xor(s, 2);
+    s += __shfl_xor(s, 4);
+    if ((c & 7u) == 0) {
+      const uint32_t g = c >> 3;
+      const _Float16 hi = (_Float16)s;
+      xs16[(size_t)m * xs_stride + g] = hi;
+      xs16[(size_t)m * xs_stride + G + g] = (_Float16)(s - (float)hi);
+    }
   }
 }
 
@@ -402,18 +399,17 @@ uint32_t xs_stride_of(const MatmulArgs& a) { return a.affine ? (2 * a.spr + KS -
 
 int blocks_of(uint32_t M) { return M <= 32 ? 1 : (M <= 64 ? 2 : 4); }
 
-// k splits: one round of workgroups over the CUs (measured: 2 beats 3 at 112 column groups on 256
-// CUs, 8 wins at 32 groups), while the f32 partial results stay small next to the weights
-// (splits x M x N x 8 bytes of extra traffic against N x K / 2)
+// k splits: one round of workgroups over the CUs for a single row tile (measured: 2 beats 3 at 112
+// column groups on 256 CUs, 8 wins at 32 groups). A function of N and K only, so that a row's
+// result does not depend on how many rows travel with it; bounded so that the f32 partial results
+// of a 32-row tile stay smaller than the weights.
 uint32_t ksplit_of(const MatmulArgs& a, const Tune& t) {
-  if (((uint64_t)a.M * a.N) % 4) return 1;  // the reduction works on groups of four outputs
+  if (a.N % 4) return 1;  // the reduction works on groups of four outputs
   if (t.skinny_ksplit > 0) return (uint32_t)t.skinny_ksplit;
-  const uint32_t rows = 32u * blocks_of(a.M);
-  const uint32_t wgs = ((a.M + rows - 1) / rows) * ((a.N + 32 * WAVES - 1) / (32 * WAVES));
+  const uint32_t ngroups = (a.N + 32 * WAVES - 1) / (32 * WAVES);
   const uint32_t nsteps = a.K / KS;
-  uint32_t want = (uint32_t)t.num_cus / wgs;
-  const uint32_t by_traffic = a.K / (16u * a.M);  // partials <= weights
-  if (want > by_traffic) want = by_traffic;
+  uint32_t want = (uint32_t)t.num_cus / ngroups;
+  if (want > a.K / 512u) want = a.K / 512u;
   if (want > 16) want = 16;
   if (want > nsteps / 4) want = nsteps / 4;
   return want < 1 ? 1 : want;
@@ -460,9 +456,8 @@ hipError_t launch_skinny(const MatmulArgs& a, const Tune& t, void* scratch, hipS
   p.ksplit = ksplit_of(a, t);
   p.steps_per_split = (p.nsteps + p.ksplit - 1) / p.ksplit;
   {
-    const uint32_t G = a.K / 64;
-    const uint32_t per_row = a.affine ? (G > p.xs_stride / 2 ? G : p.xs_stride / 2) : G;
-    const uint32_t nthr = a.M * per_row;
+    const uint32_t pad = a.affine ? p.xs_stride - 2 * (a.K / 64) : 0, cpr = a.K / 8;
+    const uint32_t nthr = a.M * (cpr > pad ? cpr : pad);  // one thread per chunk, and enough for the padding columns
     hipLaunchKernelGGL(prep_kernel, dim3((nthr + 255) / 256), dim3(256), 0, s, a.in, inp, xs16, a.M, a.K, p.xs_stride, (uint32_t)a.affine);
   }
   hipError_t e;
@@ -471,7 +466,7 @@ hipError_t launch_skinny(const MatmulArgs& a, const Tune& t, void* scratch, hipS
   else e = launch_fmt<4, false>(p, mb, s);
   if (e != hipSuccess) return e;
   if (p.ksplit > 1) {
-    const uint32_t count = a.M * a.N;  // N % 4 == 0 is checked by the caller's alignment rule on rows
+    const uint32_t count = a.M * a.N;  // N % 4 == 0 whenever ksplit > 1
     hipLaunchKernelGGL(reduce_kernel, dim3((count / 4 + 255) / 256), dim3(256), 0, s, p.partial, a.out, count, p.ksplit, (uint32_t)a.out_f32);
     return hipGetLastError();
   }
