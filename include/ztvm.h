@@ -1,7 +1,8 @@
 /*
  * libztvm_hip — C ABI of the MI355X (gfx950) int4/int3 group-quantized
  * dequant-matmul path: M=1 decode GEMV, small-M GEMV, prefill GEMM and the
- * MoE gathered GEMV.
+ * MoE gathered GEMV, plus the small dispatches either side of them in a MoE
+ * block and the load-time repack of MLX checkpoints into the bound buffers.
  *
  * The boundary it replaces is the WebGPU dispatch surface of the reference
  * engine (paths relative to the reference's root):
@@ -161,10 +162,80 @@ ZTVM_API int ztvm_matmul(ztvm_ctx* ctx, const ztvm_matmul_desc* desc);
  * and is the bit-exact parity target. */
 ZTVM_API int ztvm_dequant(ztvm_ctx* ctx, const ztvm_matmul_desc* desc);
 
+/* ---- the dispatches either side of the matmuls in an FFN / MoE block --------
+ * Each replaces one WGSL pipeline of the reference; arguments are its bindings
+ * in binding order followed by its PODArgs fields, and the token count where
+ * the reference takes it from the dispatch grid. All may be recorded. */
+
+/* silu_mul (src/compiler/shaders/silu_mul.wgsl:17-44; dispatch sites
+ * src/zero-tvm/engine-core.ts:2346, :2358, :2518): gate_up is [rows][2*ffn]
+ * f16 (gate half, then up half), out[t*ffn+i] = f16(up * gate/(1+exp(-gate)))
+ * computed in f32. rows = PODArgs.seq_len; rows == 0 dispatches nothing. */
+ZTVM_API int ztvm_silu_mul(ztvm_ctx* ctx, uint64_t out, uint64_t gate_up, uint32_t rows, uint32_t ffn);
+
+/* moe_combine (src/compiler/shaders/moe_combine.wgsl:22-44; engine-core.ts:2348):
+ * out[t*N+i] = f16(sum_s score[t*SLOTS+s] * slots[(t*SLOTS+s)*N+i]), f32
+ * accumulation in slot order. tokens = grid y. */
+ZTVM_API int ztvm_moe_combine(ztvm_ctx* ctx, uint64_t out, uint64_t slots, uint64_t score, uint32_t tokens, uint32_t N,
+                              uint32_t SLOTS);
+
+/* moe_router_logits / _q4 / _f16 (src/compiler/shaders/moe_router_logits.wgsl:30-140,
+ * moe_router_logits_f16.wgsl:20-57; engine-core.ts:2331): logits[t*rows+e] f32 =
+ * sum over groups of 64 of s*sum(x*q) + b*sum(x); bits 8 (4 values per word) or
+ * 4 (8 per word), both MLX-affine group 64; bits 16: w is [rows][D] f16 and
+ * scales/biases are ignored (pass 0). x is [tokens][D] f16. */
+ZTVM_API int ztvm_moe_router_logits(ztvm_ctx* ctx, uint64_t logits, uint64_t x, uint64_t w, uint64_t scales, uint64_t biases,
+                                    uint32_t bits, uint32_t D, uint32_t rows, uint32_t tokens);
+
+/* moe_router_topk (src/compiler/shaders/moe_router_topk.wgsl:50-136;
+ * engine-core.ts:2332): per token softmax over the E routed logits, then the K
+ * largest in descending order, ties to the lower index; scores renormalised
+ * over the survivors when norm_topk; has_shared appends slot K = (index E,
+ * sigmoid(logit E)). Strides are E+has_shared logits and K+has_shared slots per
+ * token; nothing past a token's slots is written. E <= 512, K <= min(E, 64). */
+ZTVM_API int ztvm_moe_router_topk(ztvm_ctx* ctx, uint64_t out_idx, uint64_t out_score, uint64_t logits, uint32_t E, uint32_t K,
+                                  uint32_t norm_topk, uint32_t has_shared, uint32_t tokens);
+
+/* moe_slot_translate (src/compiler/shaders/moe_slot_translate.wgsl:22-36):
+ * ids_out[i] = slot_map[ids_in[i]], a miss (0xffffffff) becomes slot 0; an id
+ * >= map_len is treated as a miss, so a bad id cannot fault the GPU. */
+ZTVM_API int ztvm_moe_slot_translate(ztvm_ctx* ctx, uint64_t ids_out, uint64_t ids_in, uint64_t slot_map, uint32_t n,
+                                     uint32_t map_len);
+
+/* ---- load-time repack of MLX safetensors records (buildBuffer) -------------
+ * The records are uploaded as they sit in the file (ztvm_upload); these calls
+ * build the bound buffers from them in device memory. `overflow` is the device
+ * address of a u32 counter (or 0): values that do not fit f16 are clamped and
+ * counted there, and the host treats a nonzero count as a hard error like the
+ * reference does (src/zero-tvm/mlx-weights.ts:533-542). */
+enum {
+  ZTVM_CONVERT_RAW = 0,      /* Convert 'raw' (mlx-weights.ts:210) */
+  ZTVM_CONVERT_BF16_F16 = 1, /* 'bf16->f16', bf16ToF16 (mlx-weights.ts:100-127) */
+  ZTVM_CONVERT_BF16_F32 = 2  /* 'bf16->f32', bf16ToF32 (mlx-weights.ts:130-135) */
+};
+
+/* One part of a concatenation plan: convert src_bytes of a record and store the
+ * result at dst, the part's place in the destination buffer
+ * (src/zero-tvm/mlx-weights.ts:490-531). bf16->f32 writes 2*src_bytes. */
+ZTVM_API int ztvm_repack_part(ztvm_ctx* ctx, uint64_t dst, uint64_t src, size_t src_bytes, int convert, uint64_t overflow);
+
+/* PlanOp permuteRows (src/zero-tvm/mlx-weights.ts:558-576): destination row j
+ * takes source row src_rows[j]. src_rows is a HOST array of src_len entries; a
+ * wrong length, bytes not divisible by rows or an index >= rows is ZTVM_E_INVALID
+ * (the reference throws). dst and src must not overlap. */
+ZTVM_API int ztvm_repack_permute_rows(ztvm_ctx* ctx, uint64_t dst, uint64_t src, size_t bytes, uint32_t rows,
+                                      const uint32_t* src_rows, uint32_t src_len);
+
+/* PlanOp dequantAffineSplit (src/zero-tvm/mlx-weights.ts:598-667): MLX-affine
+ * 4-bit group-64 [heads*(nope+v), k] -> f16 heads blocks of [k][nope] (K
+ * transposed) followed by heads blocks of [v][k]; value = fl16(fl32(q*s+b)). */
+ZTVM_API int ztvm_repack_dequant_split(ztvm_ctx* ctx, uint64_t dst, uint64_t weights, uint64_t scales, uint64_t biases,
+                                       uint32_t k, uint32_t heads, uint32_t nope, uint32_t v, uint64_t overflow);
+
 /* ---- command buffers (createCommandEncoder / finish / queue.submit) ------ */
 
-/* Between begin and end, ztvm_matmul / ztvm_dequant / ztvm_fill calls are
- * recorded instead of run (src/zero-tvm/engine-core.ts:2565-2570 records a
+/* Between begin and end, ztvm_matmul / ztvm_dequant / ztvm_fill / ztvm_copy and
+ * the block dispatches above are recorded instead of run (src/zero-tvm/engine-core.ts:2565-2570 records a
  * whole token into one encoder). Uploads, downloads and syncs are rejected
  * while recording. */
 ZTVM_API int ztvm_record_begin(ztvm_ctx* ctx);

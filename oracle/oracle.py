@@ -50,6 +50,20 @@ def lib():
                               u32p, u16p, u16p, f64p, C.c_int]
         L.zo_moe_gemv.argtypes = [C.c_int, C.c_uint32] + [C.c_uint32] * 9 + [u32p, u16p, u32p, u16p, u16p, f64p, C.c_int]
         L.zo_max_threads.restype = C.c_int
+        L.zo_bf16_to_f16.restype, L.zo_bf16_to_f16.argtypes = C.c_uint64, [u16p, u16p, C.c_size_t]
+        L.zo_bf16_to_f32.restype, L.zo_bf16_to_f32.argtypes = None, [u16p, u32p, C.c_size_t]
+        L.zo_permute_rows.argtypes = [u8p, u8p, C.c_size_t, C.c_uint32, u32p, C.c_uint32]
+        L.zo_deint.restype, L.zo_deint.argtypes = C.c_uint32, [C.c_uint32, C.c_uint32]
+        L.zo_dequant_affine_split.restype = C.c_uint64
+        L.zo_dequant_affine_split.argtypes = [u32p, u16p, u16p] + [C.c_uint32] * 4 + [u16p]
+        L.zo_silu_mul.restype, L.zo_silu_mul.argtypes = None, [u16p, C.c_uint32, C.c_uint32, f64p, u16p]
+        L.zo_moe_combine.restype = None
+        L.zo_moe_combine.argtypes = [u16p, f32p, C.c_uint32, C.c_uint32, C.c_uint32, f64p, u16p]
+        L.zo_router_logits.restype = None
+        L.zo_router_logits.argtypes = [C.c_uint32] * 4 + [u16p, C.c_void_p, u16p, u16p, f64p]
+        L.zo_router_topk.restype = None
+        L.zo_router_topk.argtypes = [f32p, C.c_uint32, C.c_uint32, C.c_uint32, C.c_int, C.c_int, u32p, f64p]
+        L.zo_slot_translate.restype, L.zo_slot_translate.argtypes = None, [u32p, u32p, C.c_uint32, u32p]
         _lib = L
     return _lib
 
@@ -145,3 +159,85 @@ def moe_gemv(mode, bits, N, K, tokens, slots, strides, ids, x, weights, scales, 
 
 def max_threads():
     return lib().zo_max_threads()
+
+
+# ---- loader conversions and the dispatches around the matmuls of a MoE block ----
+
+def bf16_to_f16(src):
+    """(f16 bit patterns, overflow count)"""
+    src = _c(src, np.uint16).ravel()
+    out = np.empty(src.size, np.uint16)
+    n = lib().zo_bf16_to_f16(_p(src, C.c_uint16), _p(out, C.c_uint16), src.size)
+    return out, int(n)
+
+
+def bf16_to_f32(src):
+    src = _c(src, np.uint16).ravel()
+    out = np.empty(src.size, np.uint32)
+    lib().zo_bf16_to_f32(_p(src, C.c_uint16), _p(out, C.c_uint32), src.size)
+    return out.view(np.float32)
+
+
+def permute_rows(data, rows, src):
+    """bytes in, bytes out; raises ValueError where the reference throws."""
+    data = np.ascontiguousarray(data).view(np.uint8).ravel()
+    src = _c(src, np.uint32).ravel()
+    out = np.empty_like(data)
+    if lib().zo_permute_rows(_p(data, C.c_uint8), _p(out, C.c_uint8), data.size, rows, _p(src, C.c_uint32), src.size):
+        raise ValueError("permuteRows: bad map, row count or index")
+    return out
+
+
+def deint(j, R):
+    return lib().zo_deint(j, R)
+
+
+def dequant_affine_split(weights, scales, biases, k, heads, nope, v):
+    """(f16 bit patterns [heads*k*nope + heads*v*k], overflow count)"""
+    w, s, b = _c(weights, np.uint32), _c(scales, np.uint16), _c(biases, np.uint16)
+    out = np.empty(heads * (nope + v) * k, np.uint16)
+    n = lib().zo_dequant_affine_split(_p(w, C.c_uint32), _p(s, C.c_uint16), _p(b, C.c_uint16), k, heads, nope, v,
+                                      _p(out, C.c_uint16))
+    return out, int(n)
+
+
+def silu_mul(gate_up, rows, ffn):
+    """(float64 unrounded [rows, ffn], f16 bit patterns of the float32 form)"""
+    gu = _c(gate_up, np.uint16)
+    o64, o16 = np.empty((rows, ffn), np.float64), np.empty((rows, ffn), np.uint16)
+    lib().zo_silu_mul(_p(gu, C.c_uint16), rows, ffn, _p(o64, C.c_double), _p(o16, C.c_uint16))
+    return o64, o16
+
+
+def moe_combine(slots, score, tokens, N, S):
+    sl, sc = _c(slots, np.uint16), _c(score, np.float32)
+    o64, o16 = np.empty((tokens, N), np.float64), np.empty((tokens, N), np.uint16)
+    lib().zo_moe_combine(_p(sl, C.c_uint16), _p(sc, C.c_float), tokens, N, S, _p(o64, C.c_double), _p(o16, C.c_uint16))
+    return o64, o16
+
+
+def router_logits(bits, D, rows, tokens, x, w, scales=None, biases=None):
+    x = _c(x, np.uint16)
+    w = _c(w, np.uint16 if bits == 16 else np.uint32)
+    s, b = _c(scales, np.uint16), _c(biases, np.uint16)
+    out = np.empty((tokens, rows), np.float64)
+    lib().zo_router_logits(bits, D, rows, tokens, _p(x, C.c_uint16), w.ctypes.data_as(C.c_void_p), _p(s, C.c_uint16),
+                           _p(b, C.c_uint16), _p(out, C.c_double))
+    return out
+
+
+def router_topk(logits, tokens, E, K, norm_topk, has_shared):
+    """(indices [tokens, K+has_shared] u32, scores float64)"""
+    lg = _c(logits, np.float32)
+    n = K + (1 if has_shared else 0)
+    idx, sc = np.empty((tokens, n), np.uint32), np.empty((tokens, n), np.float64)
+    lib().zo_router_topk(_p(lg, C.c_float), tokens, E, K, int(norm_topk), int(has_shared), _p(idx, C.c_uint32),
+                         _p(sc, C.c_double))
+    return idx, sc
+
+
+def slot_translate(ids, slot_map):
+    ids, m = _c(ids, np.uint32).ravel(), _c(slot_map, np.uint32).ravel()
+    out = np.empty_like(ids)
+    lib().zo_slot_translate(_p(ids, C.c_uint32), _p(m, C.c_uint32), ids.size, _p(out, C.c_uint32))
+    return out

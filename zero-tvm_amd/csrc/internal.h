@@ -45,6 +45,22 @@ hipError_t launch_dequant(const MatmulArgs& a, hipStream_t s);
 hipError_t launch_copy(void* dst, const void* src, size_t bytes, hipStream_t s);
 hipError_t launch_fill(void* dst, int byte, size_t bytes, hipStream_t s);
 
+// the dispatches around the matmuls of an FFN / MoE block (block_ops.hip)
+hipError_t launch_silu_mul(void* out, const void* gate_up, uint32_t rows, uint32_t ffn, hipStream_t s);
+hipError_t launch_moe_combine(void* out, const void* slots, const void* score, uint32_t tokens, uint32_t N, uint32_t S, hipStream_t s);
+hipError_t launch_router_logits(void* logits, const void* x, const void* w, const void* scales, const void* biases, uint32_t bits,
+                                uint32_t D, uint32_t rows, uint32_t tokens, hipStream_t s);
+hipError_t launch_router_topk(void* out_idx, void* out_score, const void* logits, uint32_t E, uint32_t K, uint32_t norm_topk,
+                              uint32_t has_shared, uint32_t tokens, hipStream_t s);
+uint32_t router_topk_max_experts();
+hipError_t launch_slot_translate(void* ids_out, const void* ids_in, const void* slot_map, uint32_t n, uint32_t map_len, hipStream_t s);
+
+// load-time repacking of checkpoint records (repack.hip); convert: 0 raw, 1 bf16->f16, 2 bf16->f32
+hipError_t launch_repack_convert(void* dst, const void* src, size_t src_bytes, int convert, uint32_t* counter, hipStream_t s);
+hipError_t launch_permute_rows(void* dst, const void* src, const uint32_t* map, uint32_t rows, size_t row_bytes, hipStream_t s);
+hipError_t launch_dequant_split(void* out, const void* w, const void* scales, const void* biases, uint32_t k, uint32_t heads,
+                                uint32_t nope, uint32_t v, uint32_t* counter, hipStream_t s);
+
 bool skinny_supports(const MatmulArgs& a);
 bool gemm_supports(const MatmulArgs& a);
 

@@ -25,6 +25,15 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x3 __attribute__((ext_vector_type(3)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
+// f32 -> f16 of a value that must first exist as an f32. Without the empty dependency the
+// compiler folds the producing multiply / fused multiply-add into a mixed-precision
+// instruction that rounds once, straight to f16 (and adds +0, which loses the sign of a zero
+// product); the formats here are defined as round to f32, then round to f16.
+__device__ __forceinline__ _Float16 narrow_f32(float v) {
+  asm volatile("" : "+v"(v));
+  return (_Float16)v;
+}
+
 __device__ __forceinline__ h2 as_h2(uint32_t v) { return __builtin_bit_cast(h2, v); }
 __device__ __forceinline__ uint32_t as_u32(h2 v) { return __builtin_bit_cast(uint32_t, v); }
 

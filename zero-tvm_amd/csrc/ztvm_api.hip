@@ -359,6 +359,135 @@ int ztvm_dequant(ztvm_ctx* ctx, const ztvm_matmul_desc* desc) {
   return ZTVM_OK;
 }
 
+// ---- the dispatches either side of the matmuls in an FFN / MoE block ------------------
+
+int ztvm_silu_mul(ztvm_ctx* ctx, uint64_t out, uint64_t gate_up, uint32_t rows, uint32_t ffn) {
+  if (!ctx) return fail(nullptr, ZTVM_E_INVALID, "null context");
+  if (!out || !gate_up) return fail(ctx, ZTVM_E_INVALID, "ztvm_silu_mul: null buffer");
+  if ((out | gate_up) & 1u) return fail(ctx, ZTVM_E_INVALID, "ztvm_silu_mul: buffers must be 2-byte aligned");
+  if (!ffn) return fail(ctx, ZTVM_E_INVALID, "ztvm_silu_mul: ffn must be > 0");
+  if (!rows) return ZTVM_OK;  // a zero-row chunk dispatches nothing
+  HIP_TRY(ctx, launch_silu_mul(reinterpret_cast<void*>(out), reinterpret_cast<const void*>(gate_up), rows, ffn, ctx->stream));
+  return ZTVM_OK;
+}
+
+int ztvm_moe_combine(ztvm_ctx* ctx, uint64_t out, uint64_t slots, uint64_t score, uint32_t tokens, uint32_t N, uint32_t SLOTS) {
+  if (!ctx) return fail(nullptr, ZTVM_E_INVALID, "null context");
+  if (!out || !slots || !score) return fail(ctx, ZTVM_E_INVALID, "ztvm_moe_combine: null buffer");
+  if (((out | slots) & 1u) || (score & 3u)) return fail(ctx, ZTVM_E_INVALID, "ztvm_moe_combine: misaligned buffer");
+  if (!N || !SLOTS) return fail(ctx, ZTVM_E_INVALID, "ztvm_moe_combine: N and SLOTS must be > 0");
+  if (tokens > 65535u) return fail(ctx, ZTVM_E_INVALID, "ztvm_moe_combine: at most 65535 tokens per dispatch (got %u)", tokens);
+  if (!tokens) return ZTVM_OK;
+  HIP_TRY(ctx, launch_moe_combine(reinterpret_cast<void*>(out), reinterpret_cast<const void*>(slots),
+                                  reinterpret_cast<const void*>(score), tokens, N, SLOTS, ctx->stream));
+  return ZTVM_OK;
+}
+
+int ztvm_moe_router_logits(ztvm_ctx* ctx, uint64_t logits, uint64_t x, uint64_t w, uint64_t scales, uint64_t biases, uint32_t bits,
+                           uint32_t D, uint32_t rows, uint32_t tokens) {
+  if (!ctx) return fail(nullptr, ZTVM_E_INVALID, "null context");
+  if (bits != 8 && bits != 4 && bits != 16) return fail(ctx, ZTVM_E_INVALID, "ztvm_moe_router_logits: bits must be 8, 4 or 16 (got %u)", bits);
+  if (!logits || !x || !w) return fail(ctx, ZTVM_E_INVALID, "ztvm_moe_router_logits: null buffer");
+  if (bits != 16 && (!scales || !biases)) return fail(ctx, ZTVM_E_INVALID, "ztvm_moe_router_logits: a quantized router needs scales and biases");
+  if ((x | w) & 15u) return fail(ctx, ZTVM_E_INVALID, "ztvm_moe_router_logits: x and w must be 16-byte aligned");
+  if ((logits & 3u) || ((scales | biases) & 1u)) return fail(ctx, ZTVM_E_INVALID, "ztvm_moe_router_logits: misaligned buffer");
+  if (!D || !rows) return fail(ctx, ZTVM_E_INVALID, "ztvm_moe_router_logits: D and rows must be > 0");
+  if (bits == 16 ? D % 8u : D % 64u)
+    return fail(ctx, ZTVM_E_INVALID, "ztvm_moe_router_logits: D=%u is not a multiple of %u", D, bits == 16 ? 8u : 64u);
+  if (tokens > 65535u * 8u) return fail(ctx, ZTVM_E_INVALID, "ztvm_moe_router_logits: too many tokens (%u)", tokens);
+  if (!tokens) return ZTVM_OK;
+  HIP_TRY(ctx, launch_router_logits(reinterpret_cast<void*>(logits), reinterpret_cast<const void*>(x), reinterpret_cast<const void*>(w),
+                                    reinterpret_cast<const void*>(scales), reinterpret_cast<const void*>(biases), bits, D, rows,
+                                    tokens, ctx->stream));
+  return ZTVM_OK;
+}
+
+int ztvm_moe_router_topk(ztvm_ctx* ctx, uint64_t out_idx, uint64_t out_score, uint64_t logits, uint32_t E, uint32_t K,
+                         uint32_t norm_topk, uint32_t has_shared, uint32_t tokens) {
+  if (!ctx) return fail(nullptr, ZTVM_E_INVALID, "null context");
+  if (!out_idx || !out_score || !logits) return fail(ctx, ZTVM_E_INVALID, "ztvm_moe_router_topk: null buffer");
+  if ((out_idx | out_score | logits) & 3u) return fail(ctx, ZTVM_E_INVALID, "ztvm_moe_router_topk: buffers must be 4-byte aligned");
+  if (!E || E > router_topk_max_experts())
+    return fail(ctx, ZTVM_E_INVALID, "ztvm_moe_router_topk: E must be 1..%u (got %u)", router_topk_max_experts(), E);
+  if (!K || K > E || K > 64u) return fail(ctx, ZTVM_E_INVALID, "ztvm_moe_router_topk: K must be 1..min(E, 64) (got K=%u, E=%u)", K, E);
+  if (norm_topk > 1 || has_shared > 1) return fail(ctx, ZTVM_E_INVALID, "ztvm_moe_router_topk: normTopk/hasShared must be 0 or 1");
+  if (!tokens) return ZTVM_OK;
+  HIP_TRY(ctx, launch_router_topk(reinterpret_cast<void*>(out_idx), reinterpret_cast<void*>(out_score),
+                                  reinterpret_cast<const void*>(logits), E, K, norm_topk, has_shared, tokens, ctx->stream));
+  return ZTVM_OK;
+}
+
+int ztvm_moe_slot_translate(ztvm_ctx* ctx, uint64_t ids_out, uint64_t ids_in, uint64_t slot_map, uint32_t n, uint32_t map_len) {
+  if (!ctx) return fail(nullptr, ZTVM_E_INVALID, "null context");
+  if (!ids_out || !ids_in || !slot_map) return fail(ctx, ZTVM_E_INVALID, "ztvm_moe_slot_translate: null buffer");
+  if ((ids_out | ids_in | slot_map) & 3u) return fail(ctx, ZTVM_E_INVALID, "ztvm_moe_slot_translate: buffers must be 4-byte aligned");
+  if (ids_out == ids_in) return fail(ctx, ZTVM_E_INVALID, "ztvm_moe_slot_translate: ids_in and ids_out must be separate buffers (the staging copy carries expert ids)");
+  if (!map_len) return fail(ctx, ZTVM_E_INVALID, "ztvm_moe_slot_translate: empty slot map");
+  if (!n) return ZTVM_OK;
+  HIP_TRY(ctx, launch_slot_translate(reinterpret_cast<void*>(ids_out), reinterpret_cast<const void*>(ids_in),
+                                     reinterpret_cast<const void*>(slot_map), n, map_len, ctx->stream));
+  return ZTVM_OK;
+}
+
+// ---- load-time repack ---------------------------------------------------------------------
+
+int ztvm_repack_part(ztvm_ctx* ctx, uint64_t dst, uint64_t src, size_t src_bytes, int convert, uint64_t overflow) {
+  if (!ctx) return fail(nullptr, ZTVM_E_INVALID, "null context");
+  if (convert < ZTVM_CONVERT_RAW || convert > ZTVM_CONVERT_BF16_F32) return fail(ctx, ZTVM_E_INVALID, "ztvm_repack_part: unknown convert %d", convert);
+  if (!dst || (!src && src_bytes)) return fail(ctx, ZTVM_E_INVALID, "ztvm_repack_part: null buffer");
+  if (convert != ZTVM_CONVERT_RAW) {
+    if (src_bytes & 1u) return fail(ctx, ZTVM_E_INVALID, "ztvm_repack_part: %zu bytes is not a whole number of bf16 values", src_bytes);
+    if (src & 1u) return fail(ctx, ZTVM_E_INVALID, "ztvm_repack_part: bf16 source must be 2-byte aligned");
+    if (dst & (convert == ZTVM_CONVERT_BF16_F32 ? 3u : 1u)) return fail(ctx, ZTVM_E_INVALID, "ztvm_repack_part: destination misaligned for its element type");
+  }
+  if (overflow & 3u) return fail(ctx, ZTVM_E_INVALID, "ztvm_repack_part: overflow counter must be 4-byte aligned");
+  if (!src_bytes) return ZTVM_OK;
+  HIP_TRY(ctx, launch_repack_convert(reinterpret_cast<void*>(dst), reinterpret_cast<const void*>(src), src_bytes, convert,
+                                     reinterpret_cast<uint32_t*>(overflow), ctx->stream));
+  return ZTVM_OK;
+}
+
+int ztvm_repack_permute_rows(ztvm_ctx* ctx, uint64_t dst, uint64_t src, size_t bytes, uint32_t rows, const uint32_t* src_rows,
+                             uint32_t src_len) {
+  if (!ctx) return fail(nullptr, ZTVM_E_INVALID, "null context");
+  if (!dst || !src || !src_rows) return fail(ctx, ZTVM_E_INVALID, "ztvm_repack_permute_rows: null argument");
+  if (ctx->recording) return fail(ctx, ZTVM_E_INVALID, "ztvm_repack_permute_rows while recording a command buffer");
+  if (src_len != rows) return fail(ctx, ZTVM_E_INVALID, "permuteRows has %u source indices for %u rows", src_len, rows);
+  if (!rows || bytes % rows) return fail(ctx, ZTVM_E_INVALID, "%zu B does not divide into %u rows", bytes, rows);
+  for (uint32_t j = 0; j < rows; j++)
+    if (src_rows[j] >= rows) return fail(ctx, ZTVM_E_INVALID, "permuteRows src[%u] = %u is out of range", j, src_rows[j]);
+  if ((dst < src + bytes) && (src < dst + bytes)) return fail(ctx, ZTVM_E_INVALID, "ztvm_repack_permute_rows: dst and src overlap");
+  const size_t need = (size_t)rows * 4u;
+  if (need > ctx->scratch_bytes) {
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    HIP_TRY(ctx, hipFree(ctx->scratch));
+    ctx->scratch = nullptr;
+    ctx->scratch_bytes = 0;
+    HIP_TRY(ctx, hipMalloc(&ctx->scratch, need));
+    ctx->scratch_bytes = need;
+  }
+  HIP_TRY(ctx, hipMemcpyAsync(ctx->scratch, src_rows, need, hipMemcpyHostToDevice, ctx->stream));
+  HIP_TRY(ctx, launch_permute_rows(reinterpret_cast<void*>(dst), reinterpret_cast<const void*>(src),
+                                   reinterpret_cast<const uint32_t*>(ctx->scratch), rows, bytes / rows, ctx->stream));
+  HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));  // the map may be reused on return, and the scratch by the next dispatch
+  return ZTVM_OK;
+}
+
+int ztvm_repack_dequant_split(ztvm_ctx* ctx, uint64_t dst, uint64_t weights, uint64_t scales, uint64_t biases, uint32_t k,
+                              uint32_t heads, uint32_t nope, uint32_t v, uint64_t overflow) {
+  if (!ctx) return fail(nullptr, ZTVM_E_INVALID, "null context");
+  if (!dst || !weights || !scales || !biases) return fail(ctx, ZTVM_E_INVALID, "dequantAffineSplit needs exactly [weight, scales, biases]");
+  if (!k || k % 64u) return fail(ctx, ZTVM_E_INVALID, "dequantAffineSplit: k=%u is not a multiple of the group size 64", k);
+  if (!heads || !(nope + v)) return fail(ctx, ZTVM_E_INVALID, "dequantAffineSplit: empty shape");
+  if ((uint64_t)heads * (nope + v) * (k / 8u) >= (1ull << 40)) return fail(ctx, ZTVM_E_INVALID, "dequantAffineSplit: shape too large");
+  if ((dst & 15u) || (weights & 3u) || ((scales | biases) & 1u) || (overflow & 3u))
+    return fail(ctx, ZTVM_E_INVALID, "dequantAffineSplit: misaligned buffer (dst 16, weights 4, scales/biases 2, counter 4 bytes)");
+  HIP_TRY(ctx, launch_dequant_split(reinterpret_cast<void*>(dst), reinterpret_cast<const void*>(weights),
+                                    reinterpret_cast<const void*>(scales), reinterpret_cast<const void*>(biases), k, heads, nope, v,
+                                    reinterpret_cast<uint32_t*>(overflow), ctx->stream));
+  return ZTVM_OK;
+}
+
 int ztvm_record_begin(ztvm_ctx* ctx) {
   if (!ctx) return fail(nullptr, ZTVM_E_INVALID, "null context");
   if (ctx->recording) return fail(ctx, ZTVM_E_INVALID, "already recording");

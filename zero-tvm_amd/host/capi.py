@@ -20,7 +20,10 @@ EXPORTS = [
     "ztvm_record_begin", "ztvm_record_end", "ztvm_submit", "ztvm_cmdbuf_destroy",
     "ztvm_event_create", "ztvm_event_destroy", "ztvm_event_record", "ztvm_event_elapsed_ms",
     "ztvm_set_option", "ztvm_get_option",
+    "ztvm_silu_mul", "ztvm_moe_combine", "ztvm_moe_router_logits", "ztvm_moe_router_topk", "ztvm_moe_slot_translate",
+    "ztvm_repack_part", "ztvm_repack_permute_rows", "ztvm_repack_dequant_split",
 ]
+CONVERT_RAW, CONVERT_BF16_F16, CONVERT_BF16_F32 = 0, 1, 2
 
 
 class ZtvmError(RuntimeError):
@@ -76,6 +79,15 @@ def load():
     L.ztvm_event_elapsed_ms.argtypes = [vp, vp, vp, C.POINTER(C.c_float)]
     L.ztvm_set_option.argtypes = [vp, C.c_char_p, C.c_int]
     L.ztvm_get_option.argtypes = [vp, C.c_char_p, C.POINTER(C.c_int)]
+    u32, u64 = C.c_uint32, C.c_uint64
+    L.ztvm_silu_mul.argtypes = [vp, u64, u64, u32, u32]
+    L.ztvm_moe_combine.argtypes = [vp, u64, u64, u64, u32, u32, u32]
+    L.ztvm_moe_router_logits.argtypes = [vp, u64, u64, u64, u64, u64, u32, u32, u32, u32]
+    L.ztvm_moe_router_topk.argtypes = [vp, u64, u64, u64, u32, u32, u32, u32, u32]
+    L.ztvm_moe_slot_translate.argtypes = [vp, u64, u64, u64, u32, u32]
+    L.ztvm_repack_part.argtypes = [vp, u64, u64, C.c_size_t, C.c_int, u64]
+    L.ztvm_repack_permute_rows.argtypes = [vp, u64, u64, C.c_size_t, u32, C.POINTER(u32), u32]
+    L.ztvm_repack_dequant_split.argtypes = [vp, u64, u64, u64, u64, u32, u32, u32, u32, u64]
     _lib = L
     return L
 
@@ -199,3 +211,33 @@ class Context:
         v = C.c_int()
         self._chk(self._L.ztvm_get_option(self._h, name.encode(), C.byref(v)))
         return v.value
+
+    # -- the dispatches around the matmuls of an FFN / MoE block --------------------------------
+    def silu_mul(self, out, gate_up, rows, ffn):
+        self._chk(self._L.ztvm_silu_mul(self._h, out, gate_up, rows, ffn))
+
+    def moe_combine(self, out, slots, score, tokens, N, SLOTS):
+        self._chk(self._L.ztvm_moe_combine(self._h, out, slots, score, tokens, N, SLOTS))
+
+    def moe_router_logits(self, logits, x, w, scales, biases, bits, D, rows, tokens=1):
+        self._chk(self._L.ztvm_moe_router_logits(self._h, logits, x, w, scales or 0, biases or 0, bits, D, rows, tokens))
+
+    def moe_router_topk(self, out_idx, out_score, logits, E, K, norm_topk, has_shared, tokens=1):
+        self._chk(self._L.ztvm_moe_router_topk(self._h, out_idx, out_score, logits, E, K, int(norm_topk), int(has_shared),
+                                               tokens))
+
+    def moe_slot_translate(self, ids_out, ids_in, slot_map, n, map_len):
+        self._chk(self._L.ztvm_moe_slot_translate(self._h, ids_out, ids_in, slot_map, n, map_len))
+
+    # -- load-time repack ---------------------------------------------------------------------------
+    def repack_part(self, dst, src, src_bytes, convert, overflow=0):
+        self._chk(self._L.ztvm_repack_part(self._h, dst, src, src_bytes, convert, overflow))
+
+    def repack_permute_rows(self, dst, src, nbytes, rows, src_rows):
+        import numpy as np
+        m = np.ascontiguousarray(src_rows, dtype=np.uint32)
+        self._chk(self._L.ztvm_repack_permute_rows(self._h, dst, src, nbytes, rows,
+                                                   m.ctypes.data_as(C.POINTER(C.c_uint32)), m.size))
+
+    def repack_dequant_split(self, dst, weights, scales, biases, k, heads, nope, v, overflow=0):
+        self._chk(self._L.ztvm_repack_dequant_split(self._h, dst, weights, scales, biases, k, heads, nope, v, overflow))
