@@ -281,6 +281,70 @@ def main():
             per_expert = 2 * synth.weight_bytes(ffn, d_model) + synth.weight_bytes(d_model, ffn)
             extra["moe_block_tokens%d" % tokens] = {"us": round(ms * 1e3, 2), "pairs": tokens * slots, "distinct_experts": distinct,
                                                      "expert_GB/s": round(distinct * per_expert / ms / 1e6, 1)}
+        # the whole routed FFN of configs[3] with a shared expert (257 stacked experts, 9 slots): router logits
+        # (8-bit) -> softmax top-k -> gate, up -> silu_mul -> down -> combine, routed on the device
+        E1, S = E + 1, slots + 1
+        full_w = {}
+        for name, N_, K_ in (("gate", ffn, d_model), ("up", ffn, d_model), ("down", d_model, ffn)):
+            w = synth.packed_weights(N_, K_, experts=E1, salt=10 + len(name))
+            sc = synth.scales(N_, K_, experts=E1, salt=10 + len(name))
+            bi = synth.biases(N_, K_, sc, experts=E1, salt=10 + len(name))
+            full_w[name] = tuple(_put(ctx, a) for a in (w, sc, bi))
+        rng = np.random.default_rng(17)
+        r_w = _put(ctx, rng.integers(0, 2 ** 32, (E1, d_model // 4), dtype=np.uint64).astype(np.uint32))
+        # router weights centred on zero (w = s*(q - 127.5)) so the logits are O(1) like a trained router's;
+        # logits of +-100 would push all but one probability under the f32 range and leave the top-k to ties
+        r_sh = (rng.random((E1, d_model // 64)) * 2e-4 + 2e-4).astype(np.float16)
+        r_s = _put(ctx, r_sh)
+        r_b = _put(ctx, (-127.5 * r_sh.astype(np.float32)).astype(np.float16))
+        for tokens in (1, 16):
+            xh = synth.activations(tokens, d_model, salt=6)
+            x = _put(ctx, xh)
+            logits, ids, score = ctx.alloc(tokens * E1 * 4), ctx.alloc(tokens * S * 4), ctx.alloc(tokens * S * 4)
+            gu, hbuf = ctx.alloc(tokens * S * 2 * ffn * 2), ctx.alloc(tokens * S * ffn * 2)
+            dn, y = ctx.alloc(tokens * S * d_model * 2), ctx.alloc(tokens * d_model * 2)
+            common = dict(bits=4, affine=1, M=1, slots=S, tokens=tokens, ids_stride=S, experts=E1, ids=ids)
+            dg = capi.MatmulDesc(N=ffn, k_packed=d_model // 8, scales_per_row=d_model // 64, in_slot_stride=0,
+                                 out_slot_stride=2 * ffn, in_tok_stride=d_model, out_tok_stride=S * 2 * ffn, in_=x, out=gu,
+                                 weights=full_w["gate"][0], scales=full_w["gate"][1], biases=full_w["gate"][2], **common)
+            du = capi.MatmulDesc(N=ffn, k_packed=d_model // 8, scales_per_row=d_model // 64, in_slot_stride=0,
+                                 out_slot_stride=2 * ffn, in_tok_stride=d_model, out_tok_stride=S * 2 * ffn, in_=x,
+                                 out=gu + ffn * 2, weights=full_w["up"][0], scales=full_w["up"][1], biases=full_w["up"][2], **common)
+            dd = capi.MatmulDesc(N=d_model, k_packed=ffn // 8, scales_per_row=ffn // 64, in_slot_stride=ffn,
+                                 out_slot_stride=d_model, in_tok_stride=S * ffn, out_tok_stride=S * d_model, in_=hbuf, out=dn,
+                                 weights=full_w["down"][0], scales=full_w["down"][1], biases=full_w["down"][2], **common)
+            ops = [("router_logits", lambda: ctx.moe_router_logits(logits, x, r_w, r_s, r_b, 8, d_model, E1, tokens)),
+                   ("router_topk", lambda: ctx.moe_router_topk(ids, score, logits, E, slots, True, True, tokens)),
+                   ("gate", lambda: ctx.matmul(dg)), ("up", lambda: ctx.matmul(du)),
+                   ("silu_mul", lambda: ctx.silu_mul(hbuf, gu, tokens * S, ffn)),
+                   ("down", lambda: ctx.matmul(dd)),
+                   ("combine", lambda: ctx.moe_combine(y, dn, score, tokens, d_model, S))]
+            for _, fn in ops:
+                fn()
+            # routing checked against the oracle before anything is timed
+            got_ids = ctx.download(ids, tokens * S * 4, np.uint32).reshape(tokens, S)
+            lg = ctx.download(logits, tokens * E1 * 4, np.float32).reshape(tokens, E1)
+            ref_ids, _ = oracle.router_topk(lg, tokens, E, slots, True, True)
+            yy = ctx.download(y, tokens * d_model * 2, np.float16)
+            if not np.array_equal(got_ids, ref_ids) or not np.all(np.isfinite(yy)):
+                raise SystemExit("bench: routed FFN check failed (tokens=%d)" % tokens)
+            ms = timed_graph(ctx, [fn for _ in range(20) for _, fn in ops]) / 20
+            row = {"us": round(ms * 1e3, 2), "dispatches": len(ops), "slots": S}
+            for name, fn in ops:
+                row[name + "_us"] = round(timed_graph(ctx, [fn] * 40) / 40 * 1e3, 2)
+            extra["moe_ffn_routed_tokens%d" % tokens] = row
+        # elementwise / load-time kernels at their large shapes: HBM-bound, bytes moved per second
+        rows_, f_ = 512, 14336
+        gu = ctx.alloc(rows_ * 2 * f_ * 2)
+        ho = ctx.alloc(rows_ * f_ * 2)
+        ctx.fill(gu, 0x3C, rows_ * 2 * f_ * 2)
+        ms = timed_graph(ctx, [lambda: ctx.silu_mul(ho, gu, rows_, f_)] * 20) / 20
+        extra["silu_mul_rows512_ffn14336"] = {"us": round(ms * 1e3, 2), "GB/s": round(rows_ * f_ * 6 / ms / 1e6, 1)}
+        nb = 256 << 20
+        src_, dst_ = ctx.alloc(nb), ctx.alloc(nb)
+        ctx.fill(src_, 0x3C, nb)
+        ms = timed_graph(ctx, [lambda: ctx.repack_part(dst_, src_, nb, capi.CONVERT_BF16_F16, 0)] * 6) / 6
+        extra["repack_bf16_to_f16_256MiB"] = {"us": round(ms * 1e3, 1), "GB/s": round(2 * nb / ms / 1e6, 1)}
         result["extra"] = extra
 
     if not args.no_cpu:

@@ -155,6 +155,18 @@ ZTVM_API int ztvm_matmul_resolve(const ztvm_matmul_desc* desc);
  * :4280-4293, :4386-4390). Validates, then enqueues. */
 ZTVM_API int ztvm_matmul(ztvm_ctx* ctx, const ztvm_matmul_desc* desc);
 
+/* Gate + up + SiLU in one pass over the activations: out[n] = up[n] * silu(gate[n]) with
+ * gate = W_gate x (the descriptor's weights / scales / biases) and up = W_up x (the three
+ * extra buffers, same shape and format), both sums kept in f32 until the one store.
+ * Replaces fused_ffn_kernel (src/compiler/shaders/fused_ffn.wgsl:52-140; dispatch site
+ * src/zero-tvm/engine-core.ts:2503, :2522) whose single [2*FFN, K] weight buffer is
+ * up_* = gate_* + FFN rows; with slots > 0 it runs per (token, slot) pair on expert stacks
+ * and so also replaces the gate, up and silu_mul dispatches of the MoE block
+ * (engine-core.ts:2344-2346) by one, without the f16 rounding of gate and up in between.
+ * GEMV family only (kernel AUTO or GEMV); dense M > 1 runs one pass per row. */
+ZTVM_API int ztvm_ffn_gated(ztvm_ctx* ctx, const ztvm_matmul_desc* desc, uint64_t up_weights, uint64_t up_scales,
+                            uint64_t up_biases);
+
 /* Dequantize a weight stack to [N,K] f16 (out_f32=0) or f32 (out_f32=1):
  * w = fl32(q*s + b) (or (q-7)*s), f16 = RNE of that. Uses bits, affine, N,
  * k_packed, scales_per_row, weights, scales, biases and out of `desc`.

@@ -186,7 +186,9 @@ def test_moe_block_end_to_end(ctx, capi, synth, oracle):
     S = K + 1
     rng = np.random.default_rng(3)
     x = (rng.standard_normal((tokens, D)) * 0.5).astype(np.float16)
-    rx, rw, rs, rb = router_case(8, D, E + 1, tokens, 5)
+    _, rw, rs, _ = router_case(8, D, E + 1, tokens, 5)
+    rs = (rs.astype(np.float32) * 0.02).astype(np.float16)       # centred router weights: logits of order 1,
+    rb = (-127.5 * rs.astype(np.float32)).astype(np.float16)     # so every top-k probability is far above f32 underflow
     wg, wu = synth.packed_weights((E + 1) * F, D, bits=4), synth.packed_weights((E + 1) * F, D, bits=4, salt=2)
     sg, su = synth.scales((E + 1) * F, D, affine=True), synth.scales((E + 1) * F, D, affine=True, salt=2)
     bg, bu = synth.biases((E + 1) * F, D, sg, "A"), synth.biases((E + 1) * F, D, su, "A", salt=2)
@@ -235,3 +237,85 @@ def test_moe_block_end_to_end(ctx, capi, synth, oracle):
             dn = (Wd[e] @ hh).astype(np.float16).astype(np.float64)
             ref[t] += float(rsc[t, s]) * dn
     assert np.max(np.abs(got - ref) / (np.abs(ref) + 1e-2)) < 2e-2
+
+
+# ---------------------------------------------------------------- gate + up + SiLU in one pass ---------------
+
+def gated_reference(oracle, bits, affine, N, K, x_bits, wg, sg, bg, wu, su, bu):
+    """float64: up * silu(gate) on the dequantized matrices, nothing rounded in between
+    (src/compiler/shaders/fused_ffn.wgsl:128-139 keeps both sums in f32 until the store)."""
+    Wg = oracle.dequant_matrix(bits, affine, N, K, wg, sg, bg).astype(np.float64)
+    Wu = oracle.dequant_matrix(bits, affine, N, K, wu, su, bu).astype(np.float64)
+    x = np.asarray(x_bits, np.uint16).view(np.float16).astype(np.float64)
+    g, u = x @ Wg.T, x @ Wu.T
+    return u * g / (1 + np.exp(-g))
+
+
+@pytest.mark.parametrize("bits,affine", [(4, False), (4, True), (3, True)])
+@pytest.mark.parametrize("M,N,K", [(1, 9216, 2560), (1, 100, 512), (3, 130, 1024), (1, 64, 64)])
+def test_ffn_gated_dense(ctx, capi, synth, oracle, bits, affine, M, N, K):
+    """The reference's fused FFN layout: ONE [2N, K] buffer, gate rows then up rows."""
+    x = synth.activations(M, K)
+    w = synth.packed_weights(2 * N, K, bits=bits)
+    s = synth.scales(2 * N, K, affine=affine)
+    b = synth.biases(2 * N, K, s, "A") if affine else None
+    kp, spr = K * bits // 32, K // (64 if affine else 32)
+    with Dev(ctx) as d:
+        out = d.empty((M + 1) * N * 2, fill=0)
+        W, S, B = d.put(w), d.put(s), (d.put(b) if affine else 0)
+        desc = capi.MatmulDesc(bits=bits, affine=int(affine), M=M, N=N, k_packed=kp, scales_per_row=spr, out=out, in_=d.put(x),
+                               weights=W, scales=S, biases=B)
+        ctx.ffn_gated(desc, W + N * kp * 4, S + N * spr * 2, B + N * spr * 2 if affine else 0)
+        got = ctx.download(out, (M + 1) * N * 2, np.uint16).reshape(M + 1, N)
+    ref = gated_reference(oracle, bits, affine, N, K, x, w[:N], s[:N], b[:N] if affine else None, w[N:], s[N:],
+                          b[N:] if affine else None)
+    assert np.max(np.abs(f16(got[:M]) - ref) / (np.abs(ref) + 1e-2)) < 1e-2
+    assert not got[M].any()
+
+
+def test_ffn_gated_moe_matches_three_dispatches(ctx, capi, synth, oracle):
+    """Per (token, slot) pair on expert stacks: the one-pass form against gate, up and silu_mul dispatched
+    separately (which round gate and up to f16 in between) and against the float64 formula."""
+    D, F, E, S, tokens = 512, 192, 6, 3, 4
+    x = synth.activations(tokens, D)
+    wg, wu = synth.packed_weights(E * F, D), synth.packed_weights(E * F, D, salt=2)
+    sg, su = synth.scales(E * F, D), synth.scales(E * F, D, salt=2)
+    bg, bu = synth.biases(E * F, D, sg, "B"), synth.biases(E * F, D, su, "B", salt=2)
+    ids = synth.topk_ids(tokens, S, E)
+    ids[1, 2] = 99      # a bad id: that pair is skipped by every dispatch
+    with Dev(ctx) as d:
+        X, IDS = d.put(x), d.put(ids)
+        WG, SG, BG, WU, SU, BU = (d.put(a) for a in (wg, sg, bg, wu, su, bu))
+        gate_up = d.empty(tokens * S * 2 * F * 2, fill=0)
+        h3, h1 = d.empty(tokens * S * F * 2, fill=0), d.empty(tokens * S * F * 2, fill=0)
+        common = dict(bits=4, affine=1, M=1, N=F, k_packed=D // 8, scales_per_row=D // 64, slots=S, tokens=tokens,
+                      ids=IDS, ids_stride=S, experts=E, in_=X, in_slot_stride=0, in_tok_stride=D)
+        ctx.matmul(capi.MatmulDesc(out=gate_up, out_slot_stride=2 * F, out_tok_stride=S * 2 * F, weights=WG, scales=SG, biases=BG, **common))
+        ctx.matmul(capi.MatmulDesc(out=gate_up + F * 2, out_slot_stride=2 * F, out_tok_stride=S * 2 * F, weights=WU, scales=SU, biases=BU, **common))
+        ctx.silu_mul(h3, gate_up, tokens * S, F)
+        ctx.ffn_gated(capi.MatmulDesc(out=h1, out_slot_stride=F, out_tok_stride=S * F, weights=WG, scales=SG, biases=BG, **common), WU, SU, BU)
+        a = f16(ctx.download(h3, tokens * S * F * 2, np.uint16)).reshape(tokens, S, F)
+        b = f16(ctx.download(h1, tokens * S * F * 2, np.uint16)).reshape(tokens, S, F)
+    assert not b[1, 2].any() and not a[1, 2].any()
+    assert np.max(np.abs(a - b) / (np.abs(b) + 1e-2)) < 1e-2
+    for t in range(tokens):
+        for s in range(S):
+            e = int(ids[t, s])
+            if e >= E:
+                continue
+            sl = slice(e * F, (e + 1) * F)
+            ref = gated_reference(oracle, 4, True, F, D, x[t:t + 1], wg[sl], sg[sl], bg[sl], wu[sl], su[sl], bu[sl])[0]
+            assert np.max(np.abs(b[t, s] - ref) / (np.abs(ref) + 1e-2)) < 1e-2, (t, s)
+
+
+def test_ffn_gated_rejects(ctx, capi):
+    with Dev(ctx) as d:
+        p = d.empty(1 << 16, fill=0)
+        desc = capi.MatmulDesc(bits=4, affine=1, M=1, N=64, k_packed=8, scales_per_row=1, out=p, in_=p, weights=p, scales=p, biases=p)
+        with pytest.raises(capi.ZtvmError):
+            ctx.ffn_gated(desc, p, p, 0)                       # affine without up biases
+        with pytest.raises(capi.ZtvmError):
+            ctx.ffn_gated(desc, 0, p, p)
+        desc.kernel = capi.KERNEL_GEMM
+        with pytest.raises(capi.ZtvmError):
+            ctx.ffn_gated(desc, p, p, p)

@@ -9,15 +9,32 @@
 namespace ztvm {
 namespace {
 
+// Wave-wide f32 reductions as a six-step scan over data-parallel-primitive moves (shifts within
+// rows of 16 lanes, then the two row broadcasts); lane 63 ends up with the result, which is
+// read back to every lane. The order of the additions is fixed, so results repeat exactly.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_f32(float v, float identity) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, identity), __builtin_bit_cast(int, v),
+                                                               CTRL, ROW_MASK, 0xF, false));
+}
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int m = 32; m > 0; m >>= 1) v += __shfl_xor(v, m, 64);
-  return v;
+  v += dpp_f32<0x111, 0xF>(v, 0.f);  // row_shr:1
+  v += dpp_f32<0x112, 0xF>(v, 0.f);  // row_shr:2
+  v += dpp_f32<0x114, 0xF>(v, 0.f);  // row_shr:4
+  v += dpp_f32<0x118, 0xF>(v, 0.f);  // row_shr:8
+  v += dpp_f32<0x142, 0xA>(v, 0.f);  // row_bcast:15
+  v += dpp_f32<0x143, 0xC>(v, 0.f);  // row_bcast:31
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int m = 32; m > 0; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, 64));
-  return v;
+  constexpr float LOW = -3.4e38f;
+  v = fmaxf(v, dpp_f32<0x111, 0xF>(v, LOW));
+  v = fmaxf(v, dpp_f32<0x112, 0xF>(v, LOW));
+  v = fmaxf(v, dpp_f32<0x114, 0xF>(v, LOW));
+  v = fmaxf(v, dpp_f32<0x118, 0xF>(v, LOW));
+  v = fmaxf(v, dpp_f32<0x142, 0xA>(v, LOW));
+  v = fmaxf(v, dpp_f32<0x143, 0xC>(v, LOW));
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
 // ---------------------------------------------------------------- silu_mul ----
@@ -94,11 +111,10 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(_Float16* __restrict__
 //
 // One wave per router row and per block of TT tokens: a lane reads 16 bytes of the row
 // once and uses them for every token of its block, so the row crosses L2 once per TT
-// tokens instead of once per token. Partial sums are f32; the 64 lanes are summed with
+// tokens instead of once per token. Small dispatches take TT = 1 (more waves, the work
+// is latency-bound), chunked prefill TT = 8. Partial sums are f32; the 64 lanes are summed with
 // a butterfly, so every lane (and every launch) sees the same order.
-constexpr int ROUTER_TT = 8;
-
-template <int BITS>
+template <int BITS, int ROUTER_TT>
 __global__ __launch_bounds__(256) void router_logits_kernel(float* __restrict__ logits, const _Float16* __restrict__ x,
                                                             const void* __restrict__ w, const _Float16* __restrict__ scales,
                                                             const _Float16* __restrict__ biases, uint32_t D, uint32_t rows,
@@ -165,7 +181,36 @@ __global__ __launch_bounds__(256) void router_logits_kernel(float* __restrict__ 
 // when present, is slot K with index E and sigmoid(logit[E])
 // (src/compiler/shaders/moe_router_topk.wgsl:67-136). One wave per token; lane l
 // holds experts l, l+64, ... (coalesced reads); nothing leaves registers.
+//
+// The K arg-max rounds are a serial chain, so each round is kept short: a probability and
+// its expert travel as ONE 64-bit key (f32 bits of the probability, which order like the
+// value for non-negative floats, above the complemented index, so the larger key is the
+// larger probability and, among equals, the lower index), and the wave-wide maximum is a
+// six-step scan over data-parallel-primitive moves instead of cross-lane LDS permutes.
 constexpr int TOPK_PER = 8;  // 64 lanes x 8 = 512 experts at most
+
+__device__ __forceinline__ uint64_t key_max(uint64_t a, uint64_t b) { return a > b ? a : b; }
+
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint64_t dpp_max(uint64_t v) {
+  // lanes without a source (and rows outside ROW_MASK) take 0, the identity of max over keys
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)v, CTRL, ROW_MASK, 0xF, false);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)(v >> 32), CTRL, ROW_MASK, 0xF, false);
+  return key_max(v, ((uint64_t)hi << 32) | lo);
+}
+
+// maximum of v over the 64 lanes, returned to every lane
+__device__ __forceinline__ uint64_t wave_key_max(uint64_t v) {
+  v = dpp_max<0x111, 0xF>(v);  // row_shr:1
+  v = dpp_max<0x112, 0xF>(v);  // row_shr:2
+  v = dpp_max<0x114, 0xF>(v);  // row_shr:4
+  v = dpp_max<0x118, 0xF>(v);  // row_shr:8   -> lane 15 of each row holds the row's maximum
+  v = dpp_max<0x142, 0xA>(v);  // row_bcast:15 into rows 1 and 3
+  v = dpp_max<0x143, 0xC>(v);  // row_bcast:31 into rows 2 and 3 -> lane 63 holds the wave's maximum
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, 63);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), 63);
+  return ((uint64_t)hi << 32) | lo;
+}
 
 __global__ __launch_bounds__(256) void router_topk_kernel(uint32_t* __restrict__ out_idx, float* __restrict__ out_score,
                                                           const float* __restrict__ logits, uint32_t E, uint32_t K,
@@ -184,37 +229,36 @@ __global__ __launch_bounds__(256) void router_topk_kernel(uint32_t* __restrict__
     pv[i] = e < E ? l[e] : -3.0e38f;
     m = fmaxf(m, pv[i]);
   }
+  const float shared_logit = has_shared ? l[E] : 0.f;
   const float peak = wave_max(m);
   float s = 0.f;
+  // key 0 = "no candidate": every real candidate carries a non-zero complemented index
+  uint64_t key[TOPK_PER];
 #pragma unroll
   for (int i = 0; i < TOPK_PER; i++) {
     const uint32_t e = lane + 64u * i;
-    pv[i] = e < E ? expf(pv[i] - peak) : 0.f;
-    s += pv[i];
+    const float p = e < E ? expf(pv[i] - peak) : 0.f;
+    s += p;
+    key[i] = e < E ? ((uint64_t)__builtin_bit_cast(uint32_t, p) << 32) | (0xffffffffu - e) : 0ull;
   }
   const float denom = wave_sum(s);
 
   float total = 0.f, mine = 0.f;
   uint32_t mine_idx = 0;
   for (uint32_t k = 0; k < K; k++) {
-    float bv = -1.f;
-    uint32_t bi = 0xffffffffu;
+    uint64_t best = key[0];
 #pragma unroll
-    for (int i = 0; i < TOPK_PER; i++) {
-      const uint32_t e = lane + 64u * i;
-      if (e < E && pv[i] > bv) { bv = pv[i]; bi = e; }  // ascending e within a lane: ties keep the lower index
-    }
-#pragma unroll
-    for (int sh = 32; sh > 0; sh >>= 1) {
-      const float ov = __shfl_xor(bv, sh, 64);
-      const uint32_t oi = __shfl_xor(bi, sh, 64);
-      if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-    }
+    for (int i = 1; i < TOPK_PER; i++) best = key_max(best, key[i]);
+    best = wave_key_max(best);
+    const float bv = __builtin_bit_cast(float, (uint32_t)(best >> 32));
     total += bv;
-    if (lane == k) { mine = bv; mine_idx = bi; }
+    if (lane == k) {
+      mine = bv;
+      mine_idx = 0xffffffffu - (uint32_t)best;
+    }
 #pragma unroll
     for (int i = 0; i < TOPK_PER; i++)
-      if (lane + 64u * i == bi) pv[i] = -1.f;
+      if (key[i] == best) key[i] = 0ull;  // keys are unique: exactly one register of one lane
   }
   const float scale = norm_topk ? 1.0f / total : 1.0f / denom;
   if (lane < K) {
@@ -223,7 +267,7 @@ __global__ __launch_bounds__(256) void router_topk_kernel(uint32_t* __restrict__
   }
   if (has_shared && lane == 0) {
     out_idx[obase + K] = E;
-    out_score[obase + K] = 1.0f / (1.0f + expf(-l[E]));
+    out_score[obase + K] = 1.0f / (1.0f + expf(-shared_logit));
   }
 }
 
@@ -266,16 +310,26 @@ hipError_t launch_moe_combine(void* out, const void* slots, const void* score, u
   return hipGetLastError();
 }
 
+template <int TT>
+void launch_router_tt(float* lg, const _Float16* xx, const void* w, const _Float16* sc, const _Float16* bi, uint32_t bits,
+                      uint32_t D, uint32_t rows, uint32_t tokens, hipStream_t s) {
+  const dim3 grid((rows + 3) / 4, (tokens + TT - 1) / TT);
+  if (bits == 8) hipLaunchKernelGGL((router_logits_kernel<8, TT>), grid, dim3(256), 0, s, lg, xx, w, sc, bi, D, rows, tokens);
+  else if (bits == 4) hipLaunchKernelGGL((router_logits_kernel<4, TT>), grid, dim3(256), 0, s, lg, xx, w, sc, bi, D, rows, tokens);
+  else hipLaunchKernelGGL((router_logits_kernel<16, TT>), grid, dim3(256), 0, s, lg, xx, w, sc, bi, D, rows, tokens);
+}
+
 hipError_t launch_router_logits(void* logits, const void* x, const void* w, const void* scales, const void* biases,
                                 uint32_t bits, uint32_t D, uint32_t rows, uint32_t tokens, hipStream_t s) {
-  const dim3 grid((rows + 3) / 4, (tokens + ROUTER_TT - 1) / ROUTER_TT);
   float* lg = reinterpret_cast<float*>(logits);
   const _Float16* xx = reinterpret_cast<const _Float16*>(x);
   const _Float16* sc = reinterpret_cast<const _Float16*>(scales);
   const _Float16* bi = reinterpret_cast<const _Float16*>(biases);
-  if (bits == 8) hipLaunchKernelGGL(router_logits_kernel<8>, grid, dim3(256), 0, s, lg, xx, w, sc, bi, D, rows, tokens);
-  else if (bits == 4) hipLaunchKernelGGL(router_logits_kernel<4>, grid, dim3(256), 0, s, lg, xx, w, sc, bi, D, rows, tokens);
-  else hipLaunchKernelGGL(router_logits_kernel<16>, grid, dim3(256), 0, s, lg, xx, w, sc, bi, D, rows, tokens);
+  // enough waves to cover the chip first, weight reuse second
+  const uint64_t waves1 = (uint64_t)rows * tokens;
+  if (waves1 >= 8u * 4096u) launch_router_tt<8>(lg, xx, w, sc, bi, bits, D, rows, tokens, s);
+  else if (waves1 >= 2u * 4096u) launch_router_tt<2>(lg, xx, w, sc, bi, bits, D, rows, tokens, s);
+  else launch_router_tt<1>(lg, xx, w, sc, bi, bits, D, rows, tokens, s);
   return hipGetLastError();
 }
 

@@ -32,6 +32,9 @@ struct GemvParams {
   const uint32_t* weights;
   const _Float16* biases;
   const uint32_t* ids;
+  const _Float16* scales2;   // gated form: the up projection's scales / weights / biases (same shape as the gate's)
+  const uint32_t* weights2;
+  const _Float16* biases2;
   uint32_t N, k_packed, spr, nchunks, npasses, ntiles;
   uint32_t out_f32, moe;
   uint32_t slots, in_slot_stride, out_slot_stride, in_tok_stride, out_tok_stride, ids_stride, experts;
@@ -52,12 +55,16 @@ struct Frag {
   _Float16 s[ROWS], b[ROWS];
 };
 
-template <int BITS, bool AFFINE, int LPR, int ROWS, int MAXT>
+// GATED: every row is computed twice, against the gate matrix and against the up matrix, and the
+// store is SiLU(gate) * up with both sums still in f32 (the reference's fused FFN kernel,
+// src/compiler/shaders/fused_ffn.wgsl:52-140: one pass over x, one rounding at the store).
+template <int BITS, bool AFFINE, int LPR, int ROWS, int MAXT, bool GATED = false>
 __global__ __launch_bounds__(MAXT) void gemv_kernel(const GemvParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
   constexpr int SUB = 64 / LPR;          // row slots per wave load
   constexpr int RPW = ROWS * SUB;        // rows per wave step
   constexpr int WPC = BITS == 4 ? 4 : 3; // words per chunk
+  constexpr int FR = GATED ? 2 * ROWS : ROWS;  // fragment rows: gate rows, then the same rows of the up matrix
 
   const uint32_t tid = threadIdx.x;
   const uint32_t lane = tid & 63u;
@@ -71,6 +78,9 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(const GemvParams p) {
   const uint32_t* wbase = p.weights;
   const _Float16* sbase = p.scales;
   const _Float16* bbase = p.biases;
+  const uint32_t* wbase2 = p.weights2;
+  const _Float16* sbase2 = p.scales2;
+  const _Float16* bbase2 = p.biases2;
   size_t out_base = 0;
   if (p.moe) {
     const uint32_t token = blockIdx.y / p.slots, slot = blockIdx.y % p.slots;
@@ -79,6 +89,11 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(const GemvParams p) {
     wbase += (size_t)expert * p.N * p.k_packed;
     sbase += (size_t)expert * p.N * p.spr;
     bbase += (size_t)expert * p.N * p.spr;
+    if (GATED) {
+      wbase2 += (size_t)expert * p.N * p.k_packed;
+      sbase2 += (size_t)expert * p.N * p.spr;
+      bbase2 += (size_t)expert * p.N * p.spr;
+    }
     x += (size_t)token * p.in_tok_stride + (size_t)slot * p.in_slot_stride;
     out_base = (size_t)token * p.out_tok_stride + (size_t)slot * p.out_slot_stride;
   }
@@ -88,15 +103,16 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(const GemvParams p) {
 
   // Loads of one (tile, pass). Rows past N and chunks past K are clamped to a
   // valid address (their contribution is masked later), so no lane diverges.
-  auto issue = [&](Frag<ROWS>& f, uint32_t tile, uint32_t pass) {
+  auto issue = [&](Frag<FR>& f, uint32_t tile, uint32_t pass) {
     const uint32_t c = pass * LPR + lk;
     const uint32_t cc = c < p.nchunks ? c : p.nchunks - 1;
     const uint32_t g = AFFINE ? (cc >> 1) : cc;
 #pragma unroll
-    for (int r = 0; r < ROWS; r++) {
-      uint32_t rr = tile * RPW + r * SUB + sub;
+    for (int r = 0; r < FR; r++) {
+      const bool up = GATED && r >= ROWS;
+      uint32_t rr = tile * RPW + (r % ROWS) * SUB + sub;
       rr = rr < p.N ? rr : p.N - 1;
-      const uint32_t* wp = wbase + (size_t)rr * p.k_packed + (size_t)cc * WPC;
+      const uint32_t* wp = (up ? wbase2 : wbase) + (size_t)rr * p.k_packed + (size_t)cc * WPC;
       if (BITS == 4) {
         const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp));
         f.w[r][0] = v.x; f.w[r][1] = v.y; f.w[r][2] = v.z; f.w[r][3] = v.w;
@@ -104,8 +120,8 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(const GemvParams p) {
         const words3 v = __builtin_nontemporal_load(reinterpret_cast<const words3*>(wp));
         f.w[r][0] = v.x; f.w[r][1] = v.y; f.w[r][2] = v.z; f.w[r][3] = 0;
       }
-      f.s[r] = sbase[(size_t)rr * p.spr + g];
-      if (AFFINE) f.b[r] = bbase[(size_t)rr * p.spr + g];
+      f.s[r] = (up ? sbase2 : sbase)[(size_t)rr * p.spr + g];
+      if (AFFINE) f.b[r] = (up ? bbase2 : bbase)[(size_t)rr * p.spr + g];
     }
   };
 
@@ -114,7 +130,7 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(const GemvParams p) {
   const uint32_t wave_stride = gridDim.x * waves;
   uint32_t tile = blockIdx.x * waves + wave, pass = 0;
   bool have = tile < p.ntiles;
-  Frag<ROWS> fa, fb;
+  Frag<FR> fa, fb;
   if (have) issue(fa, tile, 0);
 
   // ---- stage x: each thread converts whole chunks -------------------------
@@ -138,12 +154,12 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(const GemvParams p) {
   }
   __syncthreads();
 
-  float acc[ROWS];
+  float acc[FR];
 #pragma unroll
-  for (int r = 0; r < ROWS; r++) acc[r] = 0.f;
+  for (int r = 0; r < FR; r++) acc[r] = 0.f;
 
   // One pipeline stage: prefetch the next (tile, pass) into `nxt`, then consume `cur`.
-  auto stage = [&](const Frag<ROWS>& cur, Frag<ROWS>& nxt) {
+  auto stage = [&](const Frag<FR>& cur, Frag<FR>& nxt) {
     uint32_t ntile = tile, npass = pass + 1;
     if (npass == p.npasses) { npass = 0; ntile += wave_stride; }
     const bool nhave = ntile < p.ntiles;
@@ -166,7 +182,7 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(const GemvParams p) {
     }
     const float xs = xsum[cc];
 #pragma unroll
-    for (int r = 0; r < ROWS; r++) {
+    for (int r = 0; r < FR; r++) {
       h2 q[16];
       if (BITS == 4) unpack4_chunk(cur.w[r][0], cur.w[r][1], cur.w[r][2], cur.w[r][3], q, kc);
       else unpack3_chunk(cur.w[r][0], cur.w[r][1], cur.w[r][2], q, kc);
@@ -185,8 +201,13 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(const GemvParams p) {
     if (pass == p.npasses - 1) {
 #pragma unroll
       for (int r = 0; r < ROWS; r++) {
-        const float total = group_sum_to_last_lane<LPR>(acc[r]);
+        float total = group_sum_to_last_lane<LPR>(acc[r]);
         acc[r] = 0.f;
+        if (GATED) {
+          const float upv = group_sum_to_last_lane<LPR>(acc[r + ROWS]);
+          acc[r + ROWS] = 0.f;
+          total = upv * (total * (1.0f / (1.0f + expf(-total))));
+        }
         const uint32_t rr = tile * RPW + r * SUB + sub;
         if (lk == LPR - 1 && rr < p.N) {
           if (p.out_f32) reinterpret_cast<float*>(p.out)[out_base + rr] = total;
@@ -208,6 +229,14 @@ template <int BITS, bool AFFINE, int LPR, int ROWS>
 hipError_t launch_one(const GemvParams& p, dim3 grid, uint32_t threads, size_t smem, hipStream_t s) {
   if (threads > 512) hipLaunchKernelGGL((gemv_kernel<BITS, AFFINE, LPR, ROWS, 1024>), grid, dim3(threads), smem, s, p);
   else hipLaunchKernelGGL((gemv_kernel<BITS, AFFINE, LPR, ROWS, 512>), grid, dim3(threads), smem, s, p);
+  return hipGetLastError();
+}
+
+template <int BITS, bool AFFINE>
+hipError_t launch_gated(const GemvParams& p, int lpr, dim3 grid, uint32_t threads, size_t smem, hipStream_t s) {
+  if (lpr == 64) hipLaunchKernelGGL((gemv_kernel<BITS, AFFINE, 64, 1, 512, true>), grid, dim3(threads), smem, s, p);
+  else if (lpr == 32) hipLaunchKernelGGL((gemv_kernel<BITS, AFFINE, 32, 1, 512, true>), grid, dim3(threads), smem, s, p);
+  else hipLaunchKernelGGL((gemv_kernel<BITS, AFFINE, 16, 1, 512, true>), grid, dim3(threads), smem, s, p);
   return hipGetLastError();
 }
 
@@ -234,6 +263,8 @@ hipError_t launch_gemv(const MatmulArgs& a, const Tune& t, hipStream_t s) {
   p.slots = a.slots; p.in_slot_stride = a.in_slot_stride; p.out_slot_stride = a.out_slot_stride;
   p.in_tok_stride = a.in_tok_stride; p.out_tok_stride = a.out_tok_stride; p.ids_stride = a.ids_stride;
   p.experts = a.experts;
+  const bool gated = a.up_weights != nullptr;
+  p.weights2 = a.up_weights; p.scales2 = a.up_scales; p.biases2 = a.up_biases;
 
   // lanes per row: narrow rows share a wave between several rows
   const int lpr = p.nchunks > 32 ? 64 : (p.nchunks > 16 ? 32 : 16);
@@ -245,9 +276,10 @@ hipError_t launch_gemv(const MatmulArgs& a, const Tune& t, hipStream_t s) {
   // per wave load) use 2 steps in flight.
   const int cus = t.num_cus;
   int rows = lpr == 64 ? (t.gemv_rows ? t.gemv_rows : 1) : 2;
+  if (gated) rows = 1;  // two matrices per row already give two loads in flight
   // long rows (K >= 8192): the staged activations are 16+ KB per workgroup, so one 16-wave
   // workgroup per CU stages them once instead of three times (measured 9.4 vs 10.2 us at K=14336)
-  const bool long_rows = lpr == 64 && p.nchunks >= 256 && !p.moe;
+  const bool long_rows = lpr == 64 && p.nchunks >= 256 && !p.moe && !gated;
   uint32_t waves = t.gemv_waves ? t.gemv_waves : (long_rows ? 16 : 8);
   if (waves * 64 > (uint32_t)MAX_WG_THREADS) waves = MAX_WG_THREADS / 64;
   uint32_t gx = (uint32_t)cus * (t.gemv_wg_per_cu ? t.gemv_wg_per_cu : (long_rows ? 1 : 3));
@@ -265,6 +297,10 @@ hipError_t launch_gemv(const MatmulArgs& a, const Tune& t, hipStream_t s) {
   const uint32_t threads = waves * 64;
 
   // dense M>1 handled by the caller looping rows; here one activation row
+  if (gated) {
+    if (a.bits == 4) return a.affine ? launch_gated<4, true>(p, lpr, grid, threads, smem, s) : launch_gated<4, false>(p, lpr, grid, threads, smem, s);
+    return launch_gated<3, true>(p, lpr, grid, threads, smem, s);
+  }
   if (a.bits == 4) {
     if (a.affine) return launch_fmt<4, true>(p, lpr, rows, grid, threads, smem, s);
     return launch_fmt<4, false>(p, lpr, rows, grid, threads, smem, s);

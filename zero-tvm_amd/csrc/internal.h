@@ -13,6 +13,10 @@ struct MatmulArgs {
   const uint32_t* weights;
   const _Float16* biases;
   const uint32_t* ids;
+  // gated FFN form (null = plain matmul): the up projection, same shape and format as `weights`
+  const uint32_t* up_weights = nullptr;
+  const _Float16* up_scales = nullptr;
+  const _Float16* up_biases = nullptr;
   uint32_t M, N, K, k_packed, spr;
   uint32_t bits, affine, out_f32;
   uint32_t slots, tokens;  // slots == 0: dense

@@ -348,6 +348,31 @@ int ztvm_matmul(ztvm_ctx* ctx, const ztvm_matmul_desc* desc) {
   return ZTVM_OK;
 }
 
+int ztvm_ffn_gated(ztvm_ctx* ctx, const ztvm_matmul_desc* desc, uint64_t up_weights, uint64_t up_scales, uint64_t up_biases) {
+  if (!ctx) return fail(nullptr, ZTVM_E_INVALID, "null context");
+  char why[256];
+  int rc = validate(desc, why, sizeof why, true);
+  if (rc) return fail(ctx, rc, "ztvm_ffn_gated: %s", why);
+  if (desc->kernel != ZTVM_KERNEL_AUTO && desc->kernel != ZTVM_KERNEL_GEMV)
+    return fail(ctx, ZTVM_E_UNSUPPORTED, "ztvm_ffn_gated: kernel: only the GEMV family has the gated form");
+  if (!up_weights || !up_scales || (desc->affine && !up_biases)) return fail(ctx, ZTVM_E_INVALID, "ztvm_ffn_gated: null up-projection buffer");
+  if ((up_weights | up_scales | up_biases) & 15u) return fail(ctx, ZTVM_E_INVALID, "ztvm_ffn_gated: up-projection buffers must be 16-byte aligned");
+  MatmulArgs a = to_args(desc);
+  a.up_weights = reinterpret_cast<const uint32_t*>(up_weights);
+  a.up_scales = reinterpret_cast<const _Float16*>(up_scales);
+  a.up_biases = reinterpret_cast<const _Float16*>(up_biases);
+  const uint32_t M = a.slots ? 1 : a.M;
+  const size_t out_elt = a.out_f32 ? 4 : 2;
+  for (uint32_t m = 0; m < M; m++) {  // one pass over both matrices per activation row
+    MatmulArgs r = a;
+    r.in = a.in + (size_t)m * a.K;
+    r.out = reinterpret_cast<char*>(a.out) + (size_t)m * a.N * out_elt;
+    r.M = 1;
+    HIP_TRY(ctx, launch_gemv(r, ctx->tune, ctx->stream));
+  }
+  return ZTVM_OK;
+}
+
 int ztvm_dequant(ztvm_ctx* ctx, const ztvm_matmul_desc* desc) {
   if (!ctx) return fail(nullptr, ZTVM_E_INVALID, "null context");
   char why[256];

@@ -16,7 +16,7 @@ E_INVALID, E_HIP, E_UNSUPPORTED, E_NODEVICE = -1, -2, -3, -4
 EXPORTS = [
     "ztvm_abi_version", "ztvm_last_error", "ztvm_create", "ztvm_destroy", "ztvm_device_info",
     "ztvm_alloc", "ztvm_free", "ztvm_upload", "ztvm_download", "ztvm_fill", "ztvm_copy", "ztvm_sync",
-    "ztvm_matmul_validate", "ztvm_matmul_resolve", "ztvm_matmul", "ztvm_dequant",
+    "ztvm_matmul_validate", "ztvm_matmul_resolve", "ztvm_matmul", "ztvm_ffn_gated", "ztvm_dequant",
     "ztvm_record_begin", "ztvm_record_end", "ztvm_submit", "ztvm_cmdbuf_destroy",
     "ztvm_event_create", "ztvm_event_destroy", "ztvm_event_record", "ztvm_event_elapsed_ms",
     "ztvm_set_option", "ztvm_get_option",
@@ -80,6 +80,7 @@ def load():
     L.ztvm_set_option.argtypes = [vp, C.c_char_p, C.c_int]
     L.ztvm_get_option.argtypes = [vp, C.c_char_p, C.POINTER(C.c_int)]
     u32, u64 = C.c_uint32, C.c_uint64
+    L.ztvm_ffn_gated.argtypes = [vp, C.POINTER(MatmulDesc), u64, u64, u64]
     L.ztvm_silu_mul.argtypes = [vp, u64, u64, u32, u32]
     L.ztvm_moe_combine.argtypes = [vp, u64, u64, u64, u32, u32, u32]
     L.ztvm_moe_router_logits.argtypes = [vp, u64, u64, u64, u64, u64, u32, u32, u32, u32]
@@ -170,6 +171,9 @@ class Context:
 
     def matmul(self, desc):
         self._chk(self._L.ztvm_matmul(self._h, C.byref(desc)))
+
+    def ffn_gated(self, desc, up_weights, up_scales, up_biases=0):
+        self._chk(self._L.ztvm_ffn_gated(self._h, C.byref(desc), up_weights, up_scales, up_biases))
 
     def dequant(self, desc):
         self._chk(self._L.ztvm_dequant(self._h, C.byref(desc)))
