@@ -333,6 +333,30 @@ def main():
             for name, fn in ops:
                 row[name + "_us"] = round(timed_graph(ctx, [fn] * 40) / 40 * 1e3, 2)
             extra["moe_ffn_routed_tokens%d" % tokens] = row
+            # the same block in five launches: gate + up + SiLU in one pass over the activations
+            h2buf, dn2, y2 = ctx.alloc(tokens * S * ffn * 2), ctx.alloc(tokens * S * d_model * 2), ctx.alloc(tokens * d_model * 2)
+            dgated = capi.MatmulDesc(N=ffn, k_packed=d_model // 8, scales_per_row=d_model // 64, in_slot_stride=0,
+                                     out_slot_stride=ffn, in_tok_stride=d_model, out_tok_stride=S * ffn, in_=x, out=h2buf,
+                                     weights=full_w["gate"][0], scales=full_w["gate"][1], biases=full_w["gate"][2], **common)
+            dd2 = capi.MatmulDesc(N=d_model, k_packed=ffn // 8, scales_per_row=ffn // 64, in_slot_stride=ffn,
+                                  out_slot_stride=d_model, in_tok_stride=S * ffn, out_tok_stride=S * d_model, in_=h2buf, out=dn2,
+                                  weights=full_w["down"][0], scales=full_w["down"][1], biases=full_w["down"][2], **common)
+            fused = [ops[0], ops[1],
+                     ("gate_up_silu", lambda: ctx.ffn_gated(dgated, full_w["up"][0], full_w["up"][1], full_w["up"][2])),
+                     ("down", lambda: ctx.matmul(dd2)),
+                     ("combine", lambda: ctx.moe_combine(y2, dn2, score, tokens, d_model, S))]
+            for _, fn in fused:
+                fn()
+            y_f = ctx.download(y2, tokens * d_model * 2, np.float16).astype(np.float64)
+            y_u = yy.astype(np.float64)
+            if (not np.array_equal(ctx.download(ids, tokens * S * 4, np.uint32).reshape(tokens, S), ref_ids)
+                    or float(np.max(np.abs(y_f - y_u)) / (np.max(np.abs(y_u)) + 1e-2)) > 1e-2):  # outputs cross zero: scale by the largest
+                raise SystemExit("bench: fused routed FFN disagrees with the seven-dispatch form (tokens=%d)" % tokens)
+            ms = timed_graph(ctx, [fn for _ in range(20) for _, fn in fused]) / 20
+            row = {"us": round(ms * 1e3, 2), "dispatches": len(fused), "slots": S}
+            for name, fn in fused:
+                row[name + "_us"] = round(timed_graph(ctx, [fn] * 40) / 40 * 1e3, 2)
+            extra["moe_ffn_routed_fused_tokens%d" % tokens] = row
         # elementwise / load-time kernels at their large shapes: HBM-bound, bytes moved per second
         rows_, f_ = 512, 14336
         gu = ctx.alloc(rows_ * 2 * f_ * 2)
