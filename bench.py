@@ -237,6 +237,24 @@ def main():
         wb = synth.weight_bytes(14336, 4096, bits=3)
         extra["gemv_int3_K4096_N14336"] = {"us": round(ms * 1e3, 3), "GB/s": round(wb / ms / 1e6, 1),
                                            "hbm_frac": round(wb / ms / 1e6 / HBM_PEAK_GBS, 4)}
+        # 8-bit affine decode GEMV (int8_affine_matvec's shape family): twice the bytes per value, fewer vector
+        # instructions per byte
+        i8 = []
+        for r in range(6):
+            w = synth.packed_weights(14336, 4096, bits=8, salt=400 + r)
+            sc = synth.scales(14336, 4096, salt=400 + r)
+            bi = synth.biases(14336, 4096, sc, "A", salt=400 + r)
+            xx = synth.activations(1, 4096, salt=400 + r)
+            bufs = {"w": _put(ctx, w), "s": _put(ctx, sc), "b": _put(ctx, bi), "in": _put(ctx, xx), "out": ctx.alloc(14336 * 2)}
+            dsc = capi.MatmulDesc(bits=8, affine=1, M=1, N=14336, k_packed=4096 // 4, scales_per_row=64, out=bufs["out"],
+                                  in_=bufs["in"], scales=bufs["s"], weights=bufs["w"], biases=bufs["b"])
+            if r == 0:
+                verify(ctx, oracle, capi, dsc, (xx, w, sc, bi), 8, 4096, 14336, 1)
+            i8.append(dsc)
+        ms = timed_graph(ctx, [lambda d=i8[j % 6]: ctx.matmul(d) for j in range(120)]) / 120
+        wb = synth.weight_bytes(14336, 4096, bits=8)
+        extra["gemv_int8_K4096_N14336"] = {"us": round(ms * 1e3, 3), "GB/s": round(wb / ms / 1e6, 1),
+                                           "hbm_frac": round(wb / ms / 1e6 / HBM_PEAK_GBS, 4)}
         # small batches through the weight-streaming kernel: int4 M in {8, 32, 128} and configs[4]'s int3 M=8
         for bits, M in ((4, 8), (4, 32), (4, 128), (3, 8)):
             src = gsets if bits == 4 else None

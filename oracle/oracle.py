@@ -37,10 +37,11 @@ def lib():
         L.zo_f16_to_f32_array.argtypes = [u16p, f32p, C.c_size_t]
         L.zo_mulberry32.restype, L.zo_mulberry32.argtypes = C.c_double, [u32p]
         L.zo_reference_gemv_case.argtypes = [C.c_uint32, C.c_uint32, C.c_uint32, C.c_int, C.c_int, u16p, u16p, u16p, u32p]
-        for f in (L.zo_unpack4, L.zo_unpack3, L.zo_unpack3_window):
+        for f in (L.zo_unpack4, L.zo_unpack3, L.zo_unpack3_window, L.zo_unpack8):
             f.restype, f.argtypes = C.c_uint32, [u32p, C.c_uint32]
         L.zo_pack3.argtypes = [u8p, C.c_uint32, u32p]
         L.zo_pack4.argtypes = [u8p, C.c_uint32, u32p]
+        L.zo_pack8.argtypes = [u8p, C.c_uint32, u32p]
         L.zo_dequant_f32.restype = C.c_float
         L.zo_dequant_f32.argtypes = [C.c_uint32, C.c_uint16, C.c_uint16, C.c_int]
         L.zo_dequant_f16.restype = C.c_uint16
@@ -111,7 +112,7 @@ def reference_gemv_case(N, K, affine, q3, seed=1):
 
 def unpack(bits, row_words, k, window=False):
     row = _c(row_words, np.uint32)
-    f = lib().zo_unpack4 if bits == 4 else (lib().zo_unpack3_window if window else lib().zo_unpack3)
+    f = lib().zo_unpack4 if bits == 4 else lib().zo_unpack8 if bits == 8 else (lib().zo_unpack3_window if window else lib().zo_unpack3)
     return f(_p(row, C.c_uint32), k)
 
 
@@ -119,7 +120,7 @@ def pack(bits, values):
     v = _c(values, np.uint8).ravel()
     K = v.size
     out = np.zeros(K * bits // 32, np.uint32)
-    (lib().zo_pack3 if bits == 3 else lib().zo_pack4)(_p(v, C.c_uint8), K, _p(out, C.c_uint32))
+    (lib().zo_pack3 if bits == 3 else lib().zo_pack8 if bits == 8 else lib().zo_pack4)(_p(v, C.c_uint8), K, _p(out, C.c_uint32))
     return out
 
 

@@ -16,6 +16,7 @@
  *   zo_mulberry32                  closed-form re-derivation in Python ints
  *   zo_unpack4                     byte-wise even/odd formulation
  *                                  (int4_matmul.gen.ts:1175-1180) + numpy
+ *   zo_unpack8                     numpy's little-endian byte view of the words
  *   zo_unpack3 / zo_unpack3_window numpy.unpackbits(bitorder='little') and
  *                                  the two forms against each other for
  *                                  every block shift {0,24,16,8}
@@ -200,8 +201,17 @@ ZO_API void zo_pack4(const uint8_t* values, uint32_t K, uint32_t* words) {
   for (uint32_t i = 0; i < K; i++) words[i >> 3] |= (uint32_t)(values[i] & 15u) << (4 * (i & 7));
 }
 
+/* 8-bit (MLX affine): four unsigned bytes per word, value k at bits [8(k&3), 8(k&3)+8) of word k>>2
+ * (src/compiler/shaders/int8_affine_matvec.wgsl:57-66; tests/kernels/int8-affine.mjs:76-78). */
+ZO_API uint32_t zo_unpack8(const uint32_t* row, uint32_t k) { return (row[k >> 2] >> (8u * (k & 3u))) & 255u; }
+
+ZO_API void zo_pack8(const uint8_t* values, uint32_t K, uint32_t* words) {
+  memset(words, 0, (size_t)(K / 4) * 4);
+  for (uint32_t i = 0; i < K; i++) words[i >> 2] |= (uint32_t)values[i] << (8 * (i & 3));
+}
+
 static inline uint32_t unpack_q(const uint32_t* row, uint32_t k, uint32_t bits) {
-  return bits == 3 ? zo_unpack3(row, k) : zo_unpack4(row, k);
+  return bits == 3 ? zo_unpack3(row, k) : bits == 8 ? zo_unpack8(row, k) : zo_unpack4(row, k);
 }
 
 /* -------------------------------------------------------------- dequant -- */
@@ -250,6 +260,19 @@ ZO_API void zo_dequant_matrix(uint32_t bits, int affine, uint32_t N, uint32_t K,
 static double gemv_row_js(uint32_t bits, int affine, uint32_t K, const uint32_t* row, const uint16_t* s_row,
                           const uint16_t* b_row, const float* x) {
   double acc = 0;
+  if (bits == 8) {
+    /* the 8-bit kernels' factored form, one (scale, bias) pair per group of 64
+     * (src/compiler/shaders/int8_affine_matvec.wgsl:52-69) */
+    for (uint32_t g = 0; g < K / 64; g++) {
+      double s = zo_f16_to_f32(s_row[g]), b = zo_f16_to_f32(b_row[g]), dot = 0, xs = 0;
+      for (uint32_t i = g * 64; i < (g + 1) * 64; i++) {
+        dot += (double)x[i] * (double)zo_unpack8(row, i);
+        xs += (double)x[i];
+      }
+      acc += s * dot + b * xs;
+    }
+    return acc;
+  }
   if (bits == 3) {
     for (uint32_t i = 0; i < K; i++) {
       uint32_t g = i >> 6;

@@ -236,3 +236,27 @@ def test_moe_equals_dense_on_gathered_slab(oracle, synth):
     ids2 = np.array([[2, 2]], np.uint32)
     out = oracle.moe_gemv(oracle.MODE_FORMULA_F64, 4, N, K, 1, 2, (0, N, K, 2 * N, 2), ids2, x[:1], w, s, b, 2 * N)
     assert np.array_equal(out[:N], out[N:])
+
+
+def test_8bit_unpack_and_formula(oracle):
+    """8-bit rows: value k is byte k of the little-endian word stream; the formula mode equals a float64 matmul
+    on a matrix dequantized by numpy alone; reading the same words as 4-bit is a different matrix."""
+    rng = np.random.default_rng(8)
+    N, K, M = 12, 256, 3
+    w = rng.integers(0, 2 ** 32, (N, K // 4), dtype=np.uint64).astype(np.uint32)
+    q = w.view(np.uint8).reshape(N, K)
+    for k in (0, 1, 2, 3, 4, 63, 64, 255):
+        assert oracle.unpack(8, w[5], k) == int(q[5, k])
+    assert np.array_equal(oracle.pack(8, q[3]), w[3])
+    s = (rng.random((N, K // 64)) * 0.05 + 0.01).astype(np.float16)
+    b = (rng.random((N, K // 64)) * 0.1 - 0.05).astype(np.float16)
+    x = (rng.random((M, K)) * 2 - 1).astype(np.float16)
+    Wd = q.astype(np.float64) * np.repeat(s.astype(np.float64), 64, 1) + np.repeat(b.astype(np.float64), 64, 1)
+    want = x.astype(np.float64) @ Wd.T
+    for mode in (oracle.MODE_FORMULA_F64, oracle.MODE_JS):
+        got = oracle.gemm(mode, 8, True, M, N, K, x.view(np.uint16), w, s.view(np.uint16), b.view(np.uint16))
+        assert np.max(np.abs(got - want)) < 1e-9
+    w32 = oracle.dequant_matrix(8, True, N, K, w, s.view(np.uint16), b.view(np.uint16), want="f32")
+    assert np.array_equal(w32, (q.astype(np.float32) * np.repeat(s.astype(np.float32), 64, 1)
+                                + np.repeat(b.astype(np.float32), 64, 1)).astype(np.float32)) or \
+        np.max(np.abs(w32.astype(np.float64) - Wd) / (np.abs(Wd) + 1e-30)) < 2.0 ** -23

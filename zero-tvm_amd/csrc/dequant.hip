@@ -3,7 +3,7 @@
 // The dequantized value is the bit-exact parity target of the whole family:
 //   affine     w = fl32(q*s + b)     (src/zero-tvm/mlx-weights.ts:637-648)
 //   symmetric  w = fl32((q-7)*s)     (src/compiler/shaders/int4_matmul.gen.ts:17-19)
-// q*s is exact in f32 (<= 4 bits x 11 bits), so a single fused multiply-add
+// q*s is exact in f32 (<= 8 bits x 11 bits), so a single fused multiply-add
 // rounds once, exactly like the reference's f64 expression stored to f32.
 // The f16 form is the RNE of that f32 value (:651-660 of mlx-weights.ts).
 #include "internal.h"
@@ -36,7 +36,13 @@ __global__ __launch_bounds__(256) void dequant_kernel(const DequantParams p) {
   const float b = AFFINE ? (float)p.biases[(size_t)n * p.spr + g] : 0.f;
 
   uint32_t q[32];
-  if (BITS == 4) {
+  if (BITS == 8) {
+    const u32x4* src = reinterpret_cast<const u32x4*>(p.weights + (size_t)n * p.k_packed + (size_t)c * 8);
+    const u32x4 v0 = src[0], v1 = src[1];
+    const uint32_t w[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+    for (int i = 0; i < 32; i++) q[i] = (w[i >> 2] >> (8 * (i & 3))) & 255u;
+  } else if (BITS == 4) {
     const u32x4 v = *reinterpret_cast<const u32x4*>(p.weights + (size_t)n * p.k_packed + (size_t)c * 4);
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
@@ -117,6 +123,8 @@ hipError_t launch_dequant(const MatmulArgs& a, hipStream_t s) {
   if (a.bits == 4) {
     if (a.affine) hipLaunchKernelGGL((dequant_kernel<4, true>), grid, dim3(256), 0, s, p);
     else hipLaunchKernelGGL((dequant_kernel<4, false>), grid, dim3(256), 0, s, p);
+  } else if (a.bits == 8) {
+    hipLaunchKernelGGL((dequant_kernel<8, true>), grid, dim3(256), 0, s, p);
   } else {
     hipLaunchKernelGGL((dequant_kernel<3, true>), grid, dim3(256), 0, s, p);
   }

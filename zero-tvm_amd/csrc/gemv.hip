@@ -11,7 +11,7 @@
 //   symmetric: y = sum_chunks  s*(dot(x,q) - 7*sum(x))    (:17-19)
 //
 // Work decomposition
-//   chunk     32 consecutive k (16 B of 4-bit weights, 12 B of 3-bit): one lane-load
+//   chunk     32 consecutive k (16 B of 4-bit weights, 12 B of 3-bit, 32 B of 8-bit): one lane-load
 //   lane      owns chunk (pass*LPR + lane%LPR) of row-slot lane/LPR
 //   wave      ROWS*(64/LPR) rows per step, all passes over K, then a DPP reduce
 //   workgroup 4 waves; stages x once in LDS (slot-permuted, conflict-free
@@ -49,9 +49,9 @@ typedef uint32_t words3 __attribute__((ext_vector_type(3), aligned(4)));
 __device__ __forceinline__ uint32_t x_slot(uint32_t c, uint32_t j) { return (c >> 6) * 256u + j * 64u + (c & 63u); }
 
 // One (tile, pass) worth of global loads for ROWS rows of a wave.
-template <int ROWS>
+template <int ROWS, int WORDS>
 struct Frag {
-  uint32_t w[ROWS][4];
+  uint32_t w[ROWS][WORDS];
   _Float16 s[ROWS], b[ROWS];
 };
 
@@ -63,7 +63,8 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(const GemvParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
   constexpr int SUB = 64 / LPR;          // row slots per wave load
   constexpr int RPW = ROWS * SUB;        // rows per wave step
-  constexpr int WPC = BITS == 4 ? 4 : 3; // words per chunk
+  constexpr int WPC = BITS == 8 ? 8 : (BITS == 4 ? 4 : 3);  // words per chunk
+  constexpr int FW = BITS == 8 ? 8 : 4;                     // words a fragment row holds
   constexpr int FR = GATED ? 2 * ROWS : ROWS;  // fragment rows: gate rows, then the same rows of the up matrix
 
   const uint32_t tid = threadIdx.x;
@@ -103,7 +104,7 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(const GemvParams p) {
 
   // Loads of one (tile, pass). Rows past N and chunks past K are clamped to a
   // valid address (their contribution is masked later), so no lane diverges.
-  auto issue = [&](Frag<FR>& f, uint32_t tile, uint32_t pass) {
+  auto issue = [&](Frag<FR, FW>& f, uint32_t tile, uint32_t pass) {
     const uint32_t c = pass * LPR + lk;
     const uint32_t cc = c < p.nchunks ? c : p.nchunks - 1;
     const uint32_t g = AFFINE ? (cc >> 1) : cc;
@@ -113,7 +114,12 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(const GemvParams p) {
       uint32_t rr = tile * RPW + (r % ROWS) * SUB + sub;
       rr = rr < p.N ? rr : p.N - 1;
       const uint32_t* wp = (up ? wbase2 : wbase) + (size_t)rr * p.k_packed + (size_t)cc * WPC;
-      if (BITS == 4) {
+      if (BITS == 8) {
+        const u32x4 v0 = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp));
+        const u32x4 v1 = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp) + 1);
+        f.w[r][0] = v0.x; f.w[r][1] = v0.y; f.w[r][2] = v0.z; f.w[r][3] = v0.w;
+        f.w[r][4 % FW] = v1.x; f.w[r][5 % FW] = v1.y; f.w[r][6 % FW] = v1.z; f.w[r][7 % FW] = v1.w;
+      } else if (BITS == 4) {
         const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp));
         f.w[r][0] = v.x; f.w[r][1] = v.y; f.w[r][2] = v.z; f.w[r][3] = v.w;
       } else {
@@ -130,7 +136,7 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(const GemvParams p) {
   const uint32_t wave_stride = gridDim.x * waves;
   uint32_t tile = blockIdx.x * waves + wave, pass = 0;
   bool have = tile < p.ntiles;
-  Frag<FR> fa, fb;
+  Frag<FR, FW> fa, fb;
   if (have) issue(fa, tile, 0);
 
   // ---- stage x: each thread converts whole chunks -------------------------
@@ -145,7 +151,7 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(const GemvParams p) {
       const h8 v = src[j];
       h8 o;
 #pragma unroll
-      for (int sl = 0; sl < 8; sl++) o[sl] = v[value_in_slot(sl)];
+      for (int sl = 0; sl < 8; sl++) o[sl] = v[BITS == 8 ? value_in_slot8(sl) : value_in_slot(sl)];
       xs_pieces[x_slot(c, j)] = o;
 #pragma unroll
       for (int i = 0; i < 8; i++) s += (float)v[i];
@@ -159,7 +165,7 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(const GemvParams p) {
   for (int r = 0; r < FR; r++) acc[r] = 0.f;
 
   // One pipeline stage: prefetch the next (tile, pass) into `nxt`, then consume `cur`.
-  auto stage = [&](const Frag<FR>& cur, Frag<FR>& nxt) {
+  auto stage = [&](const Frag<FR, FW>& cur, Frag<FR, FW>& nxt) {
     uint32_t ntile = tile, npass = pass + 1;
     if (npass == p.npasses) { npass = 0; ntile += wave_stride; }
     const bool nhave = ntile < p.ntiles;
@@ -184,7 +190,8 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(const GemvParams p) {
 #pragma unroll
     for (int r = 0; r < FR; r++) {
       h2 q[16];
-      if (BITS == 4) unpack4_chunk(cur.w[r][0], cur.w[r][1], cur.w[r][2], cur.w[r][3], q, kc);
+      if constexpr (BITS == 8) unpack8_chunk(cur.w[r], q, kc);
+      else if constexpr (BITS == 4) unpack4_chunk(cur.w[r][0], cur.w[r][1], cur.w[r][2], cur.w[r][3], q, kc);
       else unpack3_chunk(cur.w[r][0], cur.w[r][1], cur.w[r][2], q, kc);
       float d0 = 0.f, d1 = 0.f;
 #pragma unroll
@@ -298,6 +305,7 @@ hipError_t launch_gemv(const MatmulArgs& a, const Tune& t, hipStream_t s) {
 
   // dense M>1 handled by the caller looping rows; here one activation row
   if (gated) {
+    if (a.bits == 8) return hipErrorInvalidValue;  // rejected by the entry point
     if (a.bits == 4) return a.affine ? launch_gated<4, true>(p, lpr, grid, threads, smem, s) : launch_gated<4, false>(p, lpr, grid, threads, smem, s);
     return launch_gated<3, true>(p, lpr, grid, threads, smem, s);
   }
@@ -305,6 +313,7 @@ hipError_t launch_gemv(const MatmulArgs& a, const Tune& t, hipStream_t s) {
     if (a.affine) return launch_fmt<4, true>(p, lpr, rows, grid, threads, smem, s);
     return launch_fmt<4, false>(p, lpr, rows, grid, threads, smem, s);
   }
+  if (a.bits == 8) return launch_fmt<8, true>(p, lpr, rows, grid, threads, smem, s);
   return launch_fmt<3, true>(p, lpr, rows, grid, threads, smem, s);
 }
 

@@ -107,6 +107,23 @@ __device__ __forceinline__ void unpack4_chunk(uint32_t w0, uint32_t w1, uint32_t
   unpack4_block(w3, q + 12, k);
 }
 
+// 8-bit values, four per word (value i at bits [8i, 8i+8)): the byte goes into the mantissa of
+// 1024, whose ulp is 1, so 1024 + q is exact for q < 1024. One word gives the pairs (v0,v2) and
+// (v1,v3); an 8-value block (two words) comes out in the slot order [v0,v2 | v1,v3 | v4,v6 | v5,v7].
+__host__ __device__ constexpr int value_in_slot8(int s) { return ((s >> 2) << 2) + ((s >> 1) & 1) + ((s & 1) << 1); }
+
+__device__ __forceinline__ void unpack8_word(uint32_t w, h2 q[2], const UnpackConsts& k) {
+  const h2 k1024 = {(_Float16)1024.f, (_Float16)1024.f};
+  q[0] = as_h2(and_or(w, 0x00FF00FFu, k.c4_lo)) - k1024;       // v0, v2
+  q[1] = as_h2(and_or(w >> 8, 0x00FF00FFu, k.c4_lo)) - k1024;  // v1, v3
+}
+
+// 32 consecutive 8-bit values = eight words
+__device__ __forceinline__ void unpack8_chunk(const uint32_t w[8], h2 q[16], const UnpackConsts& k) {
+#pragma unroll
+  for (int i = 0; i < 8; i++) unpack8_word(w[i], q + 2 * i, k);
+}
+
 // Sum over all 64 lanes (LANES=64), or over each aligned group of LANES lanes,
 // with DPP row operations. After the call the LAST lane of each group holds
 // the group's sum.

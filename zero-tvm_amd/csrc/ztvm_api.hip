@@ -63,9 +63,10 @@ void why_set(char* why, size_t n, const char* fmt, ...) {
 // about arithmetic, plus the layout contract of the bindings.
 int validate(const ztvm_matmul_desc* d, char* why, size_t n, bool need_in_out) {
   if (!d) { why_set(why, n, "null descriptor"); return ZTVM_E_INVALID; }
-  if (d->bits != 4 && d->bits != 3) { why_set(why, n, "bits must be 4 or 3 (got %u)", d->bits); return ZTVM_E_INVALID; }
+  if (d->bits != 4 && d->bits != 3 && d->bits != 8) { why_set(why, n, "bits must be 4, 3 or 8 (got %u)", d->bits); return ZTVM_E_INVALID; }
   if (d->affine > 1 || d->out_f32 > 1) { why_set(why, n, "affine/out_f32 must be 0 or 1"); return ZTVM_E_INVALID; }
   if (d->bits == 3 && !d->affine) { why_set(why, n, "q3 requires affine (3-bit ships only in the MLX-affine layout)"); return ZTVM_E_INVALID; }
+  if (d->bits == 8 && !d->affine) { why_set(why, n, "8-bit requires affine (8-bit ships only in the MLX-affine layout)"); return ZTVM_E_INVALID; }
   if (d->slots && !d->affine) { why_set(why, n, "moe requires affine (the MoE weights are MLX affine-quantised)"); return ZTVM_E_INVALID; }
   if (d->kernel > ZTVM_KERNEL_GEMM) { why_set(why, n, "unknown kernel family %u", d->kernel); return ZTVM_E_INVALID; }
   if (!d->N) { why_set(why, n, "N must be > 0"); return ZTVM_E_INVALID; }
@@ -355,6 +356,7 @@ int ztvm_ffn_gated(ztvm_ctx* ctx, const ztvm_matmul_desc* desc, uint64_t up_weig
   if (rc) return fail(ctx, rc, "ztvm_ffn_gated: %s", why);
   if (desc->kernel != ZTVM_KERNEL_AUTO && desc->kernel != ZTVM_KERNEL_GEMV)
     return fail(ctx, ZTVM_E_UNSUPPORTED, "ztvm_ffn_gated: kernel: only the GEMV family has the gated form");
+  if (desc->bits == 8) return fail(ctx, ZTVM_E_UNSUPPORTED, "ztvm_ffn_gated: no 8-bit form");
   if (!up_weights || !up_scales || (desc->affine && !up_biases)) return fail(ctx, ZTVM_E_INVALID, "ztvm_ffn_gated: null up-projection buffer");
   if ((up_weights | up_scales | up_biases) & 15u) return fail(ctx, ZTVM_E_INVALID, "ztvm_ffn_gated: up-projection buffers must be 16-byte aligned");
   MatmulArgs a = to_args(desc);

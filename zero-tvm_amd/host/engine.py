@@ -123,7 +123,11 @@ INT4_MATMUL_VARIANTS = (
 GEMM_ENTRIES = tuple(n + s for n in ("int4_matmul_tiled_m", "int4_matmul_tiled_st", "int4_matmul_sgmat",
                                      "int4_matmul_sg_e1", "int4_matmul_sg_e5") for s in ("", "_affine"))
 
-ALL_ENTRIES = tuple(int4_matmul_entry(o) for o in INT4_MATMUL_VARIANTS) + GEMM_ENTRIES
+# The 8-bit MLX-affine twins: same bindings and PODArgs, K_PACKED = K/4 (compiler.ts:429-430;
+# src/compiler/shaders/int8_affine_matvec.wgsl, int8_affine_batched.wgsl).
+INT8_ENTRIES = ("int8_affine_matvec", "int8_affine_batched")
+
+ALL_ENTRIES = tuple(int4_matmul_entry(o) for o in INT4_MATMUL_VARIANTS) + GEMM_ENTRIES + INT8_ENTRIES
 
 
 @dataclass(frozen=True)
@@ -143,6 +147,9 @@ def create_pipeline(entry):
     """compile()'s job for one entry point (compiler.ts:341-371): name -> Pipeline. Unknown names raise."""
     if entry not in ALL_ENTRIES:
         raise ValueError("unknown int4 matmul entry point '%s'" % entry)
+    if entry in INT8_ENTRIES:
+        batched = entry.endswith("_batched")
+        return Pipeline(entry, True, 8, False, False, batched, 1, capi.KERNEL_AUTO if batched else capi.KERNEL_GEMV)
     affine = "_affine" in entry
     if entry in GEMM_ENTRIES:
         # the reference's matrix-unit rungs; tiled_m / tiled_st keep f32 weights, which every family here does

@@ -38,6 +38,7 @@ export declare class Device {
 export declare const KERNEL: { AUTO: 0; GEMV: 1; SKINNY: 2; GEMM: 3 }
 export declare const INT4_MATMUL_VARIANTS: ReadonlyArray<Int4MatmulOpts>
 export declare const GEMM_ENTRIES: ReadonlyArray<string>
+export declare const INT8_ENTRIES: ReadonlyArray<string>
 export declare const ALL_ENTRIES: ReadonlyArray<string>
 export declare function int4MatmulEntry(opts?: Int4MatmulOpts): string
 export declare function checkOpts(opts?: Int4MatmulOpts): void

@@ -76,11 +76,18 @@ const GEMM_ENTRIES = []
 for (const n of ['int4_matmul_tiled_m', 'int4_matmul_tiled_st', 'int4_matmul_sgmat', 'int4_matmul_sg_e1', 'int4_matmul_sg_e5']) {
   GEMM_ENTRIES.push(n, n + '_affine')
 }
-const ALL_ENTRIES = INT4_MATMUL_VARIANTS.map(int4MatmulEntry).concat(GEMM_ENTRIES)
+// the 8-bit MLX-affine twins: same bindings and PODArgs, K_PACKED = K/4 (compiler.ts:429-430)
+const INT8_ENTRIES = ['int8_affine_matvec', 'int8_affine_batched']
+const ALL_ENTRIES = INT4_MATMUL_VARIANTS.map(int4MatmulEntry).concat(GEMM_ENTRIES, INT8_ENTRIES)
 
 /** compile()'s job for one entry point: name -> what it means for the descriptor. */
 function createPipeline(entry) {
   if (ALL_ENTRIES.indexOf(entry) < 0) throw new Error("unknown int4 matmul entry point '" + entry + "'")
+  if (INT8_ENTRIES.indexOf(entry) >= 0) {
+    const batched = /_batched$/.test(entry)
+    return Object.freeze({ label: entry, affine: true, bits: 8, outF32: false, moe: false, runtimeM: batched, fixedM: 1,
+                           kernel: batched ? KERNEL.AUTO : KERNEL.GEMV })
+  }
   const affine = entry.indexOf('_affine') >= 0
   const base = { label: entry, affine, bits: 4, outF32: false, moe: false, runtimeM: false, fixedM: 1, kernel: KERNEL.GEMV }
   if (GEMM_ENTRIES.indexOf(entry) >= 0) return Object.freeze(Object.assign(base, { runtimeM: true, kernel: KERNEL.GEMM }))
@@ -258,7 +265,7 @@ function moePods(dModel, ffn, slots, bits) {
 }
 
 module.exports = {
-  KERNEL, Device, Uniform, int4MatmulEntry, checkOpts, INT4_MATMUL_VARIANTS, GEMM_ENTRIES, ALL_ENTRIES, createPipeline,
+  KERNEL, Device, Uniform, int4MatmulEntry, checkOpts, INT4_MATMUL_VARIANTS, GEMM_ENTRIES, INT8_ENTRIES, ALL_ENTRIES, createPipeline,
   resolveMatmul, resolveChunkCap, pickChunkGemm, foldGridX, densePod, moePods,
   validate: (desc) => addon().validate(desc), resolve: (desc) => addon().resolve(desc), abiVersion: () => addon().abiVersion(),
 }
