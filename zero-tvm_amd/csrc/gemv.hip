@@ -289,6 +289,7 @@ hipError_t launch_gemv(const MatmulArgs& a, const Tune& t, hipStream_t s) {
   const bool long_rows = lpr == 64 && p.nchunks >= 256 && !p.moe && !gated;
   uint32_t waves = t.gemv_waves ? t.gemv_waves : (long_rows ? 16 : 8);
   if (waves * 64 > (uint32_t)MAX_WG_THREADS) waves = MAX_WG_THREADS / 64;
+  if (gated && waves > 8) waves = 8;  // the gated kernels are built for 512 threads
   uint32_t gx = (uint32_t)cus * (t.gemv_wg_per_cu ? t.gemv_wg_per_cu : (long_rows ? 1 : 3));
   const uint32_t rpw = rows * (64 / lpr);
   p.ntiles = (a.N + rpw - 1) / rpw;
