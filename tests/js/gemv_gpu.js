@@ -35,5 +35,32 @@ const put = (name) => { const b = load(name); const buf = dev.createBuffer(b.len
   fs.writeFileSync(path.join(dir, 'y_moe.bin'), Buffer.from(dev.readBuffer(out)))
   if (E <= 0) throw new Error('meta')
 }
+{
+  // the dispatches around the matmuls: router logits -> top-k, silu_mul, combine, gate + up + SiLU in one pass
+  const { D, E, K, rowsS, F, N2, S, GK, GF } = meta.block
+  const logits = dev.createBuffer((E + 1) * 4, 'logits'), idx = dev.createBuffer((K + 1) * 4, 'idx'), sc = dev.createBuffer((K + 1) * 4, 'score')
+  dev.moeRouterLogits(logits, put('rx.bin'), put('rw.bin'), put('rs.bin'), put('rb.bin'), 8, D, E + 1, 1)
+  dev.moeRouterTopk(idx, sc, logits, E, K, true, true, 1)
+  fs.writeFileSync(path.join(dir, 'r_logits.bin'), Buffer.from(dev.readBuffer(logits)))
+  fs.writeFileSync(path.join(dir, 'r_idx.bin'), Buffer.from(dev.readBuffer(idx)))
+  fs.writeFileSync(path.join(dir, 'r_score.bin'), Buffer.from(dev.readBuffer(sc)))
+  const h = dev.createBuffer(rowsS * F * 2, 'h')
+  dev.siluMul(h, put('gu.bin'), rowsS, F)
+  fs.writeFileSync(path.join(dir, 'h.bin'), Buffer.from(dev.readBuffer(h)))
+  const y = dev.createBuffer(N2 * 2, 'y')
+  dev.moeCombine(y, put('slots.bin'), put('cscore.bin'), 1, N2, S)
+  fs.writeFileSync(path.join(dir, 'comb.bin'), Buffer.from(dev.readBuffer(y)))
+  // the reference's fused FFN layout: one [2*GF, GK] buffer, gate rows then up rows
+  const pipe = dev.createPipeline('int4_matmul_tiled_affine')
+  const gw = put('gw.bin'), gs = put('gs.bin'), gb = put('gb.bin'), go = dev.createBuffer(GF * 2, 'gated')
+  const group = dev.bg(pipe, [go, put('gx.bin'), gs, gw, dev.uniformBuf(z.densePod(GK, GF)), gb])
+  const kp = GK / 8, spr = GK / 64
+  dev.ffnGated(pipe, group, { buffer: gw, offset: GF * kp * 4, size: GF * kp * 4 }, { buffer: gs, offset: GF * spr * 2, size: GF * spr * 2 },
+    { buffer: gb, offset: GF * spr * 2, size: GF * spr * 2 }, GF / 4)
+  fs.writeFileSync(path.join(dir, 'gated.bin'), Buffer.from(dev.readBuffer(go)))
+  let threw = false
+  try { dev.moeRouterTopk(idx, sc, logits, E, E + 1, true, true, 1) } catch (e) { threw = /K must be/.test(e.message) }
+  if (!threw) throw new Error('top-k with K > E did not throw')
+}
 dev.close()
 console.log('js gpu dispatch ok')

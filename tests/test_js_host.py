@@ -44,8 +44,25 @@ def test_js_dispatch_on_gpu(tmp_path, synth, oracle):
     ids, mx = synth.topk_ids(tokens, slots, E), synth.activations(tokens, d)
     for name, arr in (("x", x), ("w", w), ("s", s), ("b", b), ("mw", mw), ("ms", ms), ("mb", mb), ("ids", ids), ("mx", mx)):
         arr.tofile(str(tmp_path / (name + ".bin")))
+    # the block dispatches: router, silu_mul, combine, gated FFN
+    rng = np.random.default_rng(4)
+    D, RE, RK, rowsS, F, N2, S, GK, GF = 512, 16, 4, 5, 64, 96, 5, 512, 128
+    rx = (rng.random((1, D)) * 2 - 1).astype(np.float16)
+    rw = rng.integers(0, 2 ** 32, (RE + 1, D // 4), dtype=np.uint64).astype(np.uint32)
+    rs = (rng.random((RE + 1, D // 64)) * 4e-4 + 2e-4).astype(np.float16)
+    rb = (-127.5 * rs.astype(np.float32)).astype(np.float16)
+    gu = (rng.random((rowsS, 2 * F)) * 6 - 3).astype(np.float16)
+    cslots = rng.standard_normal((1, S, N2)).astype(np.float16)
+    cscore = rng.random((1, S)).astype(np.float32)
+    gx, gw, gs = synth.activations(1, GK, salt=7), synth.packed_weights(2 * GF, GK, salt=7), synth.scales(2 * GF, GK, salt=7)
+    gb = synth.biases(2 * GF, GK, gs, salt=7)
+    for name, arr in (("rx", rx), ("rw", rw), ("rs", rs), ("rb", rb), ("gu", gu), ("slots", cslots), ("cscore", cscore),
+                      ("gx", gx), ("gw", gw), ("gs", gs), ("gb", gb)):
+        arr.tofile(str(tmp_path / (name + ".bin")))
     (tmp_path / "meta.json").write_text(json.dumps({"dense": {"K": K, "N": N},
-                                                    "moe": {"E": E, "slots": slots, "tokens": tokens, "d": d, "ffn": ffn}}))
+                                                    "moe": {"E": E, "slots": slots, "tokens": tokens, "d": d, "ffn": ffn},
+                                                    "block": {"D": D, "E": RE, "K": RK, "rowsS": rowsS, "F": F, "N2": N2, "S": S,
+                                                              "GK": GK, "GF": GF}}))
     r = subprocess.run([NODE, os.path.join(ROOT, "tests", "js", "gemv_gpu.js"), str(tmp_path)], capture_output=True,
                        text=True, timeout=300)
     assert r.returncode == 0 and "js gpu dispatch ok" in r.stdout, r.stdout + r.stderr
@@ -57,3 +74,17 @@ def test_js_dispatch_on_gpu(tmp_path, synth, oracle):
                          mw, ms, mb, ym.size).reshape(tokens, slots, 2, ffn)
     assert rel_err(ym[:, :, 0], rm[:, :, 0], 1e-2) < 1e-2
     assert not ym[:, :, 1].any()  # the up half was not dispatched
+    lg = np.fromfile(str(tmp_path / "r_logits.bin"), np.float32).reshape(1, RE + 1)
+    ref_lg = oracle.router_logits(8, D, RE + 1, 1, rx.view(np.uint16), rw, rs.view(np.uint16), rb.view(np.uint16))
+    assert np.max(np.abs(lg - ref_lg)) < 1e-4
+    ri, rsc = oracle.router_topk(lg, 1, RE, RK, True, True)
+    assert np.array_equal(np.fromfile(str(tmp_path / "r_idx.bin"), np.uint32).reshape(1, RK + 1), ri)
+    assert np.max(np.abs(np.fromfile(str(tmp_path / "r_score.bin"), np.float32).reshape(1, RK + 1) - rsc)) < 2e-6
+    h64, _ = oracle.silu_mul(gu.view(np.uint16), rowsS, F)
+    assert np.max(np.abs(np.fromfile(str(tmp_path / "h.bin"), np.float16).astype(np.float64).reshape(rowsS, F) - h64)) < 5e-3
+    _, c16 = oracle.moe_combine(cslots.view(np.uint16), cscore, 1, N2, S)
+    assert np.array_equal(np.fromfile(str(tmp_path / "comb.bin"), np.uint16).reshape(1, N2), c16)
+    Wd = oracle.dequant_matrix(4, True, 2 * GF, GK, gw, gs, gb).astype(np.float64)
+    xv = gx.view(np.float16).astype(np.float64)[0]
+    g, u = Wd[:GF] @ xv, Wd[GF:] @ xv
+    assert rel_err(np.fromfile(str(tmp_path / "gated.bin"), np.float16).astype(np.float64), u * g / (1 + np.exp(-g)), 1e-2) < 1e-2

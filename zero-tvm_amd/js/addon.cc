@@ -368,13 +368,110 @@ napi_value SetOption(napi_env env, napi_callback_info info) {  // (ctx, name, va
   return undefined(env);
 }
 
+// (ctx, NA device addresses, NB u32 values): the block dispatches all have this shape
+template <size_t NA, size_t NB>
+bool get_addr_u32(napi_env env, napi_callback_info info, void** ctx, uint64_t (&addr)[NA], uint32_t (&val)[NB]) {
+  napi_value a[1 + NA + NB];
+  if (!get_args(env, info, 1 + NA + NB, a) || !get_ptr(env, a[0], ctx)) return false;
+  for (size_t i = 0; i < NA; i++)
+    if (!get_u64(env, a[1 + i], &addr[i])) return false;
+  for (size_t i = 0; i < NB; i++)
+    if (napi_get_value_uint32(env, a[1 + NA + i], &val[i]) != napi_ok) {
+      napi_throw_type_error(env, nullptr, "ztvm addon: expected a number");
+      return false;
+    }
+  return true;
+}
+
+napi_value SiluMul(napi_env env, napi_callback_info info) {  // (ctx, out, gateUp, rows, ffn)
+  void* p; uint64_t a[2]; uint32_t v[2];
+  if (!get_addr_u32(env, info, &p, a, v)) return nullptr;
+  int rc = ztvm_silu_mul((ztvm_ctx*)p, a[0], a[1], v[0], v[1]);
+  return rc ? throw_ztvm(env, (ztvm_ctx*)p, rc, "ztvm_silu_mul") : undefined(env);
+}
+
+napi_value MoeCombine(napi_env env, napi_callback_info info) {  // (ctx, out, slots, score, tokens, N, SLOTS)
+  void* p; uint64_t a[3]; uint32_t v[3];
+  if (!get_addr_u32(env, info, &p, a, v)) return nullptr;
+  int rc = ztvm_moe_combine((ztvm_ctx*)p, a[0], a[1], a[2], v[0], v[1], v[2]);
+  return rc ? throw_ztvm(env, (ztvm_ctx*)p, rc, "ztvm_moe_combine") : undefined(env);
+}
+
+napi_value MoeRouterLogits(napi_env env, napi_callback_info info) {  // (ctx, logits, x, w, scales, biases, bits, D, rows, tokens)
+  void* p; uint64_t a[5]; uint32_t v[4];
+  if (!get_addr_u32(env, info, &p, a, v)) return nullptr;
+  int rc = ztvm_moe_router_logits((ztvm_ctx*)p, a[0], a[1], a[2], a[3], a[4], v[0], v[1], v[2], v[3]);
+  return rc ? throw_ztvm(env, (ztvm_ctx*)p, rc, "ztvm_moe_router_logits") : undefined(env);
+}
+
+napi_value MoeRouterTopk(napi_env env, napi_callback_info info) {  // (ctx, outIdx, outScore, logits, E, K, normTopk, hasShared, tokens)
+  void* p; uint64_t a[3]; uint32_t v[5];
+  if (!get_addr_u32(env, info, &p, a, v)) return nullptr;
+  int rc = ztvm_moe_router_topk((ztvm_ctx*)p, a[0], a[1], a[2], v[0], v[1], v[2], v[3], v[4]);
+  return rc ? throw_ztvm(env, (ztvm_ctx*)p, rc, "ztvm_moe_router_topk") : undefined(env);
+}
+
+napi_value MoeSlotTranslate(napi_env env, napi_callback_info info) {  // (ctx, idsOut, idsIn, slotMap, n, mapLen)
+  void* p; uint64_t a[3]; uint32_t v[2];
+  if (!get_addr_u32(env, info, &p, a, v)) return nullptr;
+  int rc = ztvm_moe_slot_translate((ztvm_ctx*)p, a[0], a[1], a[2], v[0], v[1]);
+  return rc ? throw_ztvm(env, (ztvm_ctx*)p, rc, "ztvm_moe_slot_translate") : undefined(env);
+}
+
+napi_value FfnGated(napi_env env, napi_callback_info info) {  // (ctx, desc, upWeights, upScales, upBiases)
+  napi_value a[5];
+  void* p;
+  ztvm_matmul_desc d;
+  uint64_t up[3];
+  if (!get_args(env, info, 5, a) || !get_ptr(env, a[0], &p) || !get_desc(env, a[1], &d)) return nullptr;
+  for (int i = 0; i < 3; i++)
+    if (!get_u64(env, a[2 + i], &up[i])) return nullptr;
+  int rc = ztvm_ffn_gated((ztvm_ctx*)p, &d, up[0], up[1], up[2]);
+  return rc ? throw_ztvm(env, (ztvm_ctx*)p, rc, "ztvm_ffn_gated") : undefined(env);
+}
+
+napi_value RepackPart(napi_env env, napi_callback_info info) {  // (ctx, dst, src, srcBytes, convert, overflow)
+  napi_value a[6];
+  void* p;
+  uint64_t dst, src, bytes, over;
+  int32_t conv = 0;
+  if (!get_args(env, info, 6, a) || !get_ptr(env, a[0], &p) || !get_u64(env, a[1], &dst) || !get_u64(env, a[2], &src) ||
+      !get_u64(env, a[3], &bytes) || napi_get_value_int32(env, a[4], &conv) != napi_ok || !get_u64(env, a[5], &over))
+    return nullptr;
+  int rc = ztvm_repack_part((ztvm_ctx*)p, dst, src, (size_t)bytes, conv, over);
+  return rc ? throw_ztvm(env, (ztvm_ctx*)p, rc, "ztvm_repack_part") : undefined(env);
+}
+
+napi_value RepackPermuteRows(napi_env env, napi_callback_info info) {  // (ctx, dst, src, bytes, rows, Uint32Array srcRows)
+  napi_value a[6];
+  void *p, *map;
+  uint64_t dst, src, bytes;
+  uint32_t rows = 0;
+  size_t len = 0;
+  if (!get_args(env, info, 6, a) || !get_ptr(env, a[0], &p) || !get_u64(env, a[1], &dst) || !get_u64(env, a[2], &src) ||
+      !get_u64(env, a[3], &bytes) || napi_get_value_uint32(env, a[4], &rows) != napi_ok || !get_bytes(env, a[5], &map, &len))
+    return nullptr;
+  int rc = ztvm_repack_permute_rows((ztvm_ctx*)p, dst, src, (size_t)bytes, rows, (const uint32_t*)map, (uint32_t)(len / 4));
+  return rc ? throw_ztvm(env, (ztvm_ctx*)p, rc, "ztvm_repack_permute_rows") : undefined(env);
+}
+
+napi_value RepackDequantSplit(napi_env env, napi_callback_info info) {  // (ctx, dst, weights, scales, biases, overflow, k, heads, nope, v)
+  void* p; uint64_t a[5]; uint32_t v[4];
+  if (!get_addr_u32(env, info, &p, a, v)) return nullptr;
+  int rc = ztvm_repack_dequant_split((ztvm_ctx*)p, a[0], a[1], a[2], a[3], v[0], v[1], v[2], v[3], a[4]);
+  return rc ? throw_ztvm(env, (ztvm_ctx*)p, rc, "ztvm_repack_dequant_split") : undefined(env);
+}
+
 napi_value Init(napi_env env, napi_value exports) {
   struct E { const char* name; napi_callback fn; };
   static const E table[] = {
       {"abiVersion", AbiVersion}, {"create", Create}, {"destroy", Destroy}, {"deviceInfo", DeviceInfo}, {"alloc", Alloc},
       {"free", Free}, {"upload", Upload}, {"download", Download}, {"fill", Fill}, {"copy", Copy}, {"sync", Sync},
       {"validate", Validate}, {"resolve", Resolve}, {"matmul", Matmul}, {"dequant", Dequant}, {"recordBegin", RecordBegin},
-      {"recordEnd", RecordEnd}, {"submit", Submit}, {"cmdbufDestroy", CmdbufDestroy}, {"setOption", SetOption}};
+      {"recordEnd", RecordEnd}, {"submit", Submit}, {"cmdbufDestroy", CmdbufDestroy}, {"setOption", SetOption},
+      {"siluMul", SiluMul}, {"moeCombine", MoeCombine}, {"moeRouterLogits", MoeRouterLogits}, {"moeRouterTopk", MoeRouterTopk},
+      {"moeSlotTranslate", MoeSlotTranslate}, {"ffnGated", FfnGated}, {"repackPart", RepackPart},
+      {"repackPermuteRows", RepackPermuteRows}, {"repackDequantSplit", RepackDequantSplit}};
   for (const E& e : table) {
     napi_value fn;
     if (napi_create_function(env, e.name, NAPI_AUTO_LENGTH, e.fn, nullptr, &fn) != napi_ok) return nullptr;

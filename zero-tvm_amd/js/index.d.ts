@@ -4,7 +4,7 @@ export interface Int4MatmulOpts {
   mDyn?: boolean; affine?: boolean; moe?: boolean; q3?: boolean
 }
 export interface Pipeline {
-  readonly label: string; readonly affine: boolean; readonly bits: 3 | 4; readonly outF32: boolean
+  readonly label: string; readonly affine: boolean; readonly bits: 3 | 4 | 8; readonly outF32: boolean
   readonly moe: boolean; readonly runtimeM: boolean; readonly fixedM: number; readonly kernel: number
 }
 export interface MatmulDesc {
@@ -30,6 +30,15 @@ export declare class Device {
   bg(pipeline: Pipeline, bufs: BindEntry[]): BindGroup
   descriptor(group: BindGroup, wgX?: number, wgY?: number, wgZ?: number): MatmulDesc
   dispatch(pipeline: Pipeline, group: BindGroup, wgX: number, wgY?: number, wgZ?: number): void
+  siluMul(out: BindEntry, gateUp: BindEntry, rows: number, ffn: number): void
+  moeCombine(out: BindEntry, slots: BindEntry, score: BindEntry, tokens: number, N: number, SLOTS: number): void
+  moeRouterLogits(logits: BindEntry, x: BindEntry, w: BindEntry, scales: BindEntry | null, biases: BindEntry | null,
+    bits: 4 | 8 | 16, D: number, rows: number, tokens?: number): void
+  moeRouterTopk(outIdx: BindEntry, outScore: BindEntry, logits: BindEntry, E: number, K: number, normTopk: boolean,
+    hasShared: boolean, tokens?: number): void
+  moeSlotTranslate(idsOut: BindEntry, idsIn: BindEntry, slotMap: BindEntry, n: number, mapLen: number): void
+  ffnGated(pipeline: Pipeline, group: BindGroup, upWeights: BindEntry, upScales: BindEntry, upBiases: BindEntry | null,
+    wgX?: number, wgY?: number, wgZ?: number): void
   beginEncoder(): void
   finishEncoder(): unknown
   submit(cmdbuf: unknown): void

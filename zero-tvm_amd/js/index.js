@@ -244,6 +244,27 @@ class Device {
     if (d.M === 0 && !pipeline.moe) return
     addon().matmul(this.ctx, d)
   }
+  // ---- the dispatches either side of the matmuls (bindings in binding order, then the PODArgs fields, then tokens) ----
+  _a(b) { return b ? (b.buffer ? b.buffer.addr + BigInt(b.offset) : b.addr) : 0n }
+  /** silu_mul.wgsl: out [rows, ffn] <- gateUp [rows, 2*ffn] */
+  siluMul(out, gateUp, rows, ffn) { addon().siluMul(this.ctx, this._a(out), this._a(gateUp), rows, ffn) }
+  /** moe_combine.wgsl */
+  moeCombine(out, slots, score, tokens, N, SLOTS) { addon().moeCombine(this.ctx, this._a(out), this._a(slots), this._a(score), tokens, N, SLOTS) }
+  /** moe_router_logits / _q4 / _f16 by bits = 8 / 4 / 16 (scales and biases null for 16) */
+  moeRouterLogits(logits, x, w, scales, biases, bits, D, rows, tokens) {
+    addon().moeRouterLogits(this.ctx, this._a(logits), this._a(x), this._a(w), this._a(scales), this._a(biases), bits, D, rows, tokens === undefined ? 1 : tokens)
+  }
+  /** moe_router_topk.wgsl */
+  moeRouterTopk(outIdx, outScore, logits, E, K, normTopk, hasShared, tokens) {
+    addon().moeRouterTopk(this.ctx, this._a(outIdx), this._a(outScore), this._a(logits), E, K, normTopk ? 1 : 0, hasShared ? 1 : 0, tokens === undefined ? 1 : tokens)
+  }
+  /** moe_slot_translate.wgsl */
+  moeSlotTranslate(idsOut, idsIn, slotMap, n, mapLen) { addon().moeSlotTranslate(this.ctx, this._a(idsOut), this._a(idsIn), this._a(slotMap), n, mapLen) }
+  /** gate + up + SiLU in one pass: the gate's bind group and grid, plus the up projection's weights / scales / biases */
+  ffnGated(pipeline, group, upWeights, upScales, upBiases, wgX, wgY, wgZ) {
+    if (group.pipeline !== pipeline) throw new Error("ffnGated: bind group was built for '" + group.pipeline.label + "', not '" + pipeline.label + "'")
+    addon().ffnGated(this.ctx, this.descriptor(group, wgX, wgY, wgZ), this._a(upWeights), this._a(upScales), this._a(upBiases))
+  }
   beginEncoder() { addon().recordBegin(this.ctx) }
   finishEncoder() { return addon().recordEnd(this.ctx) }
   submit(cmdbuf) { addon().submit(this.ctx, cmdbuf) }
