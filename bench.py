@@ -255,6 +255,25 @@ def main():
         wb = synth.weight_bytes(14336, 4096, bits=8)
         extra["gemv_int8_K4096_N14336"] = {"us": round(ms * 1e3, 3), "GB/s": round(wb / ms / 1e6, 1),
                                            "hbm_frac": round(wb / ms / 1e6 / HBM_PEAK_GBS, 4)}
+        # QKV matmul + RoPE + KV append in one dispatch at the configs[1] qkv shape (32 heads, 8 KV heads of 128 = 6144 rows)
+        qs = []
+        hps, vpo, kps = 16 * 128, 8 * 16 * 128, 2 * 8 * 16 * 128
+        kvbuf, qout = ctx.alloc(64 * kps * 2), ctx.alloc(4096 * 2)
+        ctx.fill(kvbuf, 0, 64 * kps * 2)
+        pmap = _put(ctx, np.array([517], np.int32))
+        for r in range(8):
+            d0 = sets[r % args.sets][2]   # the (4096 -> 6144) weight set of the headline
+            qs.append(capi.QkvFusedDesc(bits=4, affine=1, k_packed=512, scales_per_row=64, heads=32, kv_heads=8, head_dim=128,
+                                        page_size=16, kv_page_stride=kps, head_page_stride=hps, v_page_offset=vpo,
+                                        rope_theta=500000.0, kv_capacity=64 * kps, q_out=qout, kv_pages=kvbuf, hidden=d0.in_,
+                                        scales=d0.scales, weights=d0.weights, position_map=pmap, biases=d0.biases))
+        ctx.qkv_fused(qs[0])
+        if not np.all(np.isfinite(ctx.download(qout, 4096 * 2, np.float16))):
+            raise SystemExit("bench: fused QKV check failed")
+        ms = timed_graph(ctx, [lambda d=qs[j % 8]: ctx.qkv_fused(d) for j in range(160)]) / 160
+        wb = synth.weight_bytes(6144, 4096)
+        extra["qkv_fused_rope_kvappend_K4096_N6144"] = {"us": round(ms * 1e3, 3), "GB/s": round(wb / ms / 1e6, 1),
+                                                        "hbm_frac": round(wb / ms / 1e6 / HBM_PEAK_GBS, 4)}
         # small batches through the weight-streaming kernel: int4 M in {8, 32, 128} and configs[4]'s int3 M=8
         for bits, M in ((4, 8), (4, 32), (4, 128), (3, 8)):
             src = gsets if bits == 4 else None

@@ -167,6 +167,32 @@ ZTVM_API int ztvm_matmul(ztvm_ctx* ctx, const ztvm_matmul_desc* desc);
 ZTVM_API int ztvm_ffn_gated(ztvm_ctx* ctx, const ztvm_matmul_desc* desc, uint64_t up_weights, uint64_t up_scales,
                             uint64_t up_biases);
 
+/* QKV matmul + RoPE + KV append in one dispatch, decode path (one token). Replaces
+ * qkv_fused / _sg / _sg_vec4 / _tiled_sg / _tiled2sg (src/compiler/shaders/qkv_fused.wgsl:23-193;
+ * dispatch site src/zero-tvm/engine-core.ts:2320): bindings 0 q_out, 1 kv_pages, 2 hidden,
+ * 3 scales, 4 weights, 5 position_map, PODArgs {position_map_elem_offset, pages_elem_offset},
+ * and the model constants the reference injects as a shader prelude
+ * (src/compiler/shader-prelude.ts:43-52). The fused projection is [Q | K | V] rows, Q =
+ * heads*head_dim, K = V = kv_heads*head_dim; for every rotary pair (dim, dim + head_dim/2) of a
+ * head the two rows are multiplied in one pass, Q and K are rotated by
+ * freq = position / theta^(2*dim/head_dim) (cos and sin in f32), Q goes to q_out, K and V into
+ * the page the position falls in: element page*kv_page_stride + head*head_page_stride +
+ * slot*head_dim + dim (+ v_page_offset for V) + pages_elem_offset. The position is read on
+ * the device from position_map[position_map_elem_offset]. A position whose slot would lie at
+ * or past kv_capacity (f16 elements; 0 = unchecked) or below zero writes Q only, so a bad
+ * position cannot fault the GPU. 4-bit rows, symmetric (the reference's) or affine. */
+typedef struct ztvm_qkv_fused_desc {
+  uint32_t bits, affine;
+  uint32_t k_packed, scales_per_row;
+  uint32_t heads, kv_heads, head_dim;
+  uint32_t page_size, kv_page_stride, head_page_stride, v_page_offset; /* f16 elements */
+  uint32_t position_map_elem_offset, pages_elem_offset;
+  float rope_theta;
+  uint64_t kv_capacity;
+  uint64_t q_out, kv_pages, hidden, scales, weights, position_map, biases;
+} ztvm_qkv_fused_desc;
+ZTVM_API int ztvm_qkv_fused(ztvm_ctx* ctx, const ztvm_qkv_fused_desc* desc);
+
 /* Dequantize a weight stack to [N,K] f16 (out_f32=0) or f32 (out_f32=1):
  * w = fl32(q*s + b) (or (q-7)*s), f16 = RNE of that. Uses bits, affine, N,
  * k_packed, scales_per_row, weights, scales, biases and out of `desc`.

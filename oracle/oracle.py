@@ -65,6 +65,8 @@ def lib():
         L.zo_router_topk.restype = None
         L.zo_router_topk.argtypes = [f32p, C.c_uint32, C.c_uint32, C.c_uint32, C.c_int, C.c_int, u32p, f64p]
         L.zo_slot_translate.restype, L.zo_slot_translate.argtypes = None, [u32p, u32p, C.c_uint32, u32p]
+        L.zo_qkv_fused.restype = None
+        L.zo_qkv_fused.argtypes = [C.c_uint32] * 10 + [C.c_double, C.c_int32, u16p, u32p, u16p, u16p, u16p, u16p]
         _lib = L
     return _lib
 
@@ -242,3 +244,15 @@ def slot_translate(ids, slot_map):
     out = np.empty_like(ids)
     lib().zo_slot_translate(_p(ids, C.c_uint32), _p(m, C.c_uint32), ids.size, _p(out, C.c_uint32))
     return out
+
+
+def qkv_fused(affine, K, heads, kv_heads, head_dim, page_size, kv_page_stride, head_page_stride, v_page_offset,
+              pages_elem_offset, theta, position, hidden, weights, scales, biases, pages):
+    """(q_out f16 bits [heads*head_dim], pages f16 bits with the token's K and V written in)"""
+    h, w, s, b = _c(hidden, np.uint16), _c(weights, np.uint32), _c(scales, np.uint16), _c(biases, np.uint16)
+    q_out = np.zeros(heads * head_dim, np.uint16)
+    pg = np.array(pages, np.uint16, copy=True)
+    lib().zo_qkv_fused(int(affine), K, heads, kv_heads, head_dim, page_size, kv_page_stride, head_page_stride, v_page_offset,
+                       pages_elem_offset, float(theta), int(position), _p(h, C.c_uint16), _p(w, C.c_uint32),
+                       _p(s, C.c_uint16), _p(b, C.c_uint16), _p(q_out, C.c_uint16), _p(pg, C.c_uint16))
+    return q_out, pg

@@ -28,6 +28,10 @@
  *   zo_router_topk          scipy softmax + stable argsort; ties, K == E,
  *                           shared slot == expit(logit[E])
  *   zo_slot_translate       numpy take + where
+ *   zo_qkv_fused            the pinned dequant + a numpy matmul, the rotation as a complex
+ *                           multiplication by exp(i*freq), the cache as a reshaped
+ *                           [page][K|V][kv_head][slot][dim] array; swapping the pair or the
+ *                           sign of the sine, or writing V rotated, fails it
  * The reference's byte-exact repack fixtures (.weights-local/kernel-refs) are
  * git-ignored and absent, so fidelity of the plans to a real MLX checkpoint is
  * "parity unpinned"; what is pinned is each conversion against numpy.
@@ -262,5 +266,53 @@ ZO_API void zo_slot_translate(const uint32_t* ids_in, const uint32_t* slot_map, 
   for (uint32_t i = 0; i < n; i++) {
     uint32_t s = slot_map[ids_in[i]];
     ids_out[i] = s == 0xffffffffu ? 0u : s;
+  }
+}
+
+/* ------------------------------------------------------------ qkv_fused -- */
+
+/* QKV matmul + RoPE + paged KV append for one token (src/compiler/shaders/qkv_fused.wgsl:41-193),
+ * following the reference test's float64 form (tests/kernels/run.mjs:797-806, :836-860):
+ * row dot products in float64 over per-element (q-7)*s (or q*s+b), freq = pos / theta^(2*dim/head_dim),
+ * rot_lo = c*lo - s*hi, rot_hi = c*hi + s*lo, everything rounded to f16 only at the store.
+ * q_out [heads*head_dim] and pages (already holding the cache's previous contents) are f16 bit patterns. */
+ZO_API void zo_qkv_fused(uint32_t affine, uint32_t K, uint32_t heads, uint32_t kv_heads, uint32_t head_dim,
+                         uint32_t page_size, uint32_t kv_page_stride, uint32_t head_page_stride, uint32_t v_page_offset,
+                         uint32_t pages_elem_offset, double theta, int32_t position, const uint16_t* hidden,
+                         const uint32_t* weights, const uint16_t* scales, const uint16_t* biases, uint16_t* q_out,
+                         uint16_t* pages) {
+  const uint32_t half = head_dim / 2, KP = K / 8, G = affine ? 64 : 32, SPR = K / G;
+  const uint32_t q_dim = heads * head_dim, kv_dim = kv_heads * head_dim;
+  const uint32_t page_no = (uint32_t)position / page_size, slot = (uint32_t)position % page_size;
+  for (uint32_t group = 0; group < 3; group++) {
+    const uint32_t nheads = group == 0 ? heads : kv_heads;
+    const uint32_t row_base = group == 0 ? 0 : group == 1 ? q_dim : q_dim + kv_dim;
+    for (uint32_t h = 0; h < nheads; h++)
+      for (uint32_t d = 0; d < half; d++) {
+        double v[2];
+        for (int part = 0; part < 2; part++) {
+          const size_t row = (size_t)row_base + (size_t)h * head_dim + d + (part ? half : 0);
+          double acc = 0;
+          for (uint32_t k = 0; k < K; k++) {
+            const uint32_t q = (weights[row * KP + (k >> 3)] >> (4 * (k & 7))) & 15u;
+            const double s = zo_f16_to_f32(scales[row * SPR + k / G]);
+            const double w = affine ? (double)q * s + (double)zo_f16_to_f32(biases[row * SPR + k / G]) : ((double)q - 7.0) * s;
+            acc += (double)zo_f16_to_f32(hidden[k]) * w;
+          }
+          v[part] = acc;
+        }
+        double lo = v[0], hi = v[1];
+        if (group != 2) {
+          const double freq = (double)position / pow(theta, (double)(d * 2) / (double)head_dim);
+          const double c = cos(freq), s = sin(freq);
+          lo = c * v[0] - s * v[1];
+          hi = c * v[1] + s * v[0];
+        }
+        uint16_t* dst = group == 0 ? q_out + (size_t)h * head_dim + d
+                                   : pages + (size_t)page_no * kv_page_stride + (size_t)h * head_page_stride +
+                                         (size_t)slot * head_dim + pages_elem_offset + d + (group == 2 ? v_page_offset : 0);
+        dst[0] = zo_f32_to_f16((float)lo);
+        dst[half] = zo_f32_to_f16((float)hi);
+      }
   }
 }

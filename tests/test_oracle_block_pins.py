@@ -224,3 +224,43 @@ def test_slot_translate(oracle):
     got = oracle.slot_translate(ids, m)
     t = m[ids]
     assert np.array_equal(got, np.where(t == 0xFFFFFFFF, 0, t))
+
+
+# ---------------------------------------------------------------- qkv_fused ----------------------------------
+
+@pytest.mark.parametrize("affine", [False, True])
+def test_qkv_fused(oracle, synth, affine):
+    """Against numpy alone: dequantized matrix @ x, the rotary pair (lo, hi) as the complex number lo + i*hi
+    multiplied by exp(i*freq), and the cache viewed as [page][K|V][kv_head][slot][dim]."""
+    heads, kv_heads, hd, K, page, pos, theta = 4, 2, 16, 128, 8, 13, 10000.0
+    half = hd // 2
+    rows = (heads + 2 * kv_heads) * hd
+    hps, vpo, kps = page * hd, kv_heads * page * hd, 2 * kv_heads * page * hd
+    x = synth.activations(1, K)
+    w = synth.packed_weights(rows, K)
+    s = synth.scales(rows, K, affine=affine)
+    b = synth.biases(rows, K, s, "A") if affine else None
+    pages0 = np.full(3 * kps, 0x1234, np.uint16)
+    q16, pg = oracle.qkv_fused(affine, K, heads, kv_heads, hd, page, kps, hps, vpo, 0, theta, pos, x, w, s, b, pages0)
+    W = oracle.dequant_matrix(4, affine, rows, K, w, s, b).astype(np.float64)
+    y = W @ x.view(np.float16).astype(np.float64)[0]
+    q, k, v = (y[:heads * hd].reshape(heads, hd), y[heads * hd:(heads + kv_heads) * hd].reshape(kv_heads, hd),
+               y[(heads + kv_heads) * hd:].reshape(kv_heads, hd))
+    rot = np.exp(1j * pos / theta ** (np.arange(half) * 2 / hd))
+
+    def rope(t):
+        z = (t[:, :half] + 1j * t[:, half:]) * rot
+        return np.concatenate([z.real, z.imag], 1)
+
+    def close(bits, want):
+        got = np.asarray(bits, np.uint16).view(np.float16).astype(np.float64)
+        return np.all(np.abs(got - want) <= np.maximum(np.abs(want), 2.0 ** -14) * 2.0 ** -10 * 0.51 + 1e-9)
+
+    assert close(q16.reshape(heads, hd), rope(q))
+    cache = pg.reshape(3, 2, kv_heads, page, hd)
+    assert close(cache[pos // page, 0, :, pos % page], rope(k))
+    assert close(cache[pos // page, 1, :, pos % page], v), "V is appended unrotated"
+    untouched = np.ones(cache.shape[:4], bool)
+    untouched[pos // page, :, :, pos % page] = False
+    assert np.all(cache[untouched] == 0x1234), "only the position's slot is written"
+    assert not close(q16.reshape(heads, hd), np.concatenate([rope(q)[:, half:], rope(q)[:, :half]], 1))

@@ -35,6 +35,14 @@ struct GemvParams {
   const _Float16* scales2;   // gated form: the up projection's scales / weights / biases (same shape as the gate's)
   const uint32_t* weights2;
   const _Float16* biases2;
+  // QKV form: rows are RoPE pairs; the epilogue rotates and scatters into q_out / the paged KV cache
+  _Float16* q_out;
+  _Float16* kv_pages;
+  const int32_t* position_map;
+  uint32_t half_dim, head_dim, q_pairs, kv_pairs, q_dim, kv_dim;
+  uint32_t page_size, kv_page_stride, head_page_stride, v_page_offset, pos_off, pages_off;
+  uint64_t kv_capacity;  // f16 elements in kv_pages; a position whose slot lies past it is not written (0 = unchecked)
+  float rope_theta;
   uint32_t N, k_packed, spr, nchunks, npasses, ntiles;
   uint32_t out_f32, moe;
   uint32_t slots, in_slot_stride, out_slot_stride, in_tok_stride, out_tok_stride, ids_stride, experts;
@@ -58,7 +66,29 @@ struct Frag {
 // GATED: every row is computed twice, against the gate matrix and against the up matrix, and the
 // store is SiLU(gate) * up with both sums still in f32 (the reference's fused FFN kernel,
 // src/compiler/shaders/fused_ffn.wgsl:52-140: one pass over x, one rounding at the store).
-template <int BITS, bool AFFINE, int LPR, int ROWS, int MAXT, bool GATED = false>
+//
+// QKV (a GATED launch whose second matrix is the first one shifted by half a head): "row" p is a
+// rotary pair of the fused Q|K|V projection, rows row_lo(p) and row_lo(p) + half_dim of the same
+// head. The pair is rotated in registers and written straight to q_out (Q) or into the paged KV
+// cache (K rotated, V as is): QKV matmul + RoPE + KV append in one dispatch
+// (src/compiler/shaders/qkv_fused.wgsl:41-193).
+struct QkvPair {
+  uint32_t group, head, dim_lo, row_lo;
+};
+__device__ __forceinline__ QkvPair qkv_pair(const GemvParams& p, uint32_t pair) {
+  QkvPair r{0u, 0u, 0u, 0u};
+  uint32_t in_group = pair, row_base = 0;
+  if (in_group >= p.q_pairs) {
+    r.group = 1; in_group -= p.q_pairs; row_base = p.q_dim;
+    if (in_group >= p.kv_pairs) { r.group = 2; in_group -= p.kv_pairs; row_base = p.q_dim + p.kv_dim; }
+  }
+  r.head = in_group / p.half_dim;
+  r.dim_lo = in_group - r.head * p.half_dim;
+  r.row_lo = row_base + r.head * p.head_dim + r.dim_lo;
+  return r;
+}
+
+template <int BITS, bool AFFINE, int LPR, int ROWS, int MAXT, bool GATED = false, bool QKV = false>
 __global__ __launch_bounds__(MAXT) void gemv_kernel(const GemvParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
   constexpr int SUB = 64 / LPR;          // row slots per wave load
@@ -113,6 +143,7 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(const GemvParams p) {
       const bool up = GATED && r >= ROWS;
       uint32_t rr = tile * RPW + (r % ROWS) * SUB + sub;
       rr = rr < p.N ? rr : p.N - 1;
+      if (QKV) rr = qkv_pair(p, rr).row_lo;
       const uint32_t* wp = (up ? wbase2 : wbase) + (size_t)rr * p.k_packed + (size_t)cc * WPC;
       if (BITS == 8) {
         const u32x4 v0 = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp));
@@ -157,6 +188,17 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(const GemvParams p) {
       for (int i = 0; i < 8; i++) s += (float)v[i];
     }
     xsum[c] = s;
+  }
+  // QKV: the rotation of every pair index, once per workgroup, by the threads at the far end of the
+  // workgroup (the staging above keeps the first ones busy); cos and sin are long instruction
+  // sequences that would otherwise run once per pair with one lane active
+  float2* rope = reinterpret_cast<float2*>(smem + (size_t)padded_chunks * 68u);
+  if (QKV) {
+    const uint32_t rt = blockDim.x - 1u - tid;
+    if (rt < p.half_dim) {
+      const float freq = (float)p.position_map[p.pos_off] / powf(p.rope_theta, (float)(rt * 2u) / (float)p.head_dim);
+      rope[rt] = float2{cosf(freq), sinf(freq)};
+    }
   }
   __syncthreads();
 
@@ -210,12 +252,35 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(const GemvParams p) {
       for (int r = 0; r < ROWS; r++) {
         float total = group_sum_to_last_lane<LPR>(acc[r]);
         acc[r] = 0.f;
+        float second = 0.f;
         if (GATED) {
-          const float upv = group_sum_to_last_lane<LPR>(acc[r + ROWS]);
+          second = group_sum_to_last_lane<LPR>(acc[r + ROWS]);
           acc[r + ROWS] = 0.f;
-          total = upv * (total * (1.0f / (1.0f + expf(-total))));
+          if (!QKV) total = second * (total * (1.0f / (1.0f + expf(-total))));
         }
         const uint32_t rr = tile * RPW + r * SUB + sub;
+        if (QKV) {
+          if (lk == LPR - 1 && rr < p.N) {
+            const QkvPair q = qkv_pair(p, rr);
+            const int position = p.position_map[p.pos_off];
+            const uint32_t page_no = (uint32_t)position / p.page_size, slot = (uint32_t)position - page_no * p.page_size;
+            const size_t cache = (size_t)page_no * p.kv_page_stride + (size_t)q.head * p.head_page_stride +
+                                 (size_t)slot * p.head_dim + p.pages_off + q.dim_lo;
+            float lo = total, hi = second;  // V: no rotation
+            if (q.group != 2) {
+              const float c = rope[q.dim_lo].x, sn = rope[q.dim_lo].y;
+              lo = c * total + sn * (-second);
+              hi = c * second + sn * total;
+            }
+            const size_t at = cache + (q.group == 2 ? p.v_page_offset : 0u);
+            _Float16* dst = q.group == 0 ? p.q_out + (size_t)q.head * p.head_dim + q.dim_lo : p.kv_pages + at;
+            if (q.group == 0 || position >= 0 && (!p.kv_capacity || at + p.half_dim < p.kv_capacity)) {
+              dst[0] = (_Float16)lo;
+              dst[p.half_dim] = (_Float16)hi;
+            }
+          }
+          continue;
+        }
         if (lk == LPR - 1 && rr < p.N) {
           if (p.out_f32) reinterpret_cast<float*>(p.out)[out_base + rr] = total;
           else reinterpret_cast<_Float16*>(p.out)[out_base + rr] = (_Float16)total;
@@ -236,6 +301,14 @@ template <int BITS, bool AFFINE, int LPR, int ROWS>
 hipError_t launch_one(const GemvParams& p, dim3 grid, uint32_t threads, size_t smem, hipStream_t s) {
   if (threads > 512) hipLaunchKernelGGL((gemv_kernel<BITS, AFFINE, LPR, ROWS, 1024>), grid, dim3(threads), smem, s, p);
   else hipLaunchKernelGGL((gemv_kernel<BITS, AFFINE, LPR, ROWS, 512>), grid, dim3(threads), smem, s, p);
+  return hipGetLastError();
+}
+
+template <int BITS, bool AFFINE>
+hipError_t launch_qkv(const GemvParams& p, int lpr, dim3 grid, uint32_t threads, size_t smem, hipStream_t s) {
+  if (lpr == 64) hipLaunchKernelGGL((gemv_kernel<BITS, AFFINE, 64, 1, 512, true, true>), grid, dim3(threads), smem, s, p);
+  else if (lpr == 32) hipLaunchKernelGGL((gemv_kernel<BITS, AFFINE, 32, 1, 512, true, true>), grid, dim3(threads), smem, s, p);
+  else hipLaunchKernelGGL((gemv_kernel<BITS, AFFINE, 16, 1, 512, true, true>), grid, dim3(threads), smem, s, p);
   return hipGetLastError();
 }
 
@@ -272,6 +345,16 @@ hipError_t launch_gemv(const MatmulArgs& a, const Tune& t, hipStream_t s) {
   p.experts = a.experts;
   const bool gated = a.up_weights != nullptr;
   p.weights2 = a.up_weights; p.scales2 = a.up_scales; p.biases2 = a.up_biases;
+  if (a.qkv) {
+    const QkvArgs& q = *a.qkv;
+    p.q_out = q.q_out; p.kv_pages = q.kv_pages; p.position_map = q.position_map;
+    p.half_dim = q.head_dim / 2; p.head_dim = q.head_dim;
+    p.q_pairs = q.heads * p.half_dim; p.kv_pairs = q.kv_heads * p.half_dim;
+    p.q_dim = q.heads * q.head_dim; p.kv_dim = q.kv_heads * q.head_dim;
+    p.page_size = q.page_size; p.kv_page_stride = q.kv_page_stride; p.head_page_stride = q.head_page_stride;
+    p.v_page_offset = q.v_page_offset; p.pos_off = q.position_map_elem_offset; p.pages_off = q.pages_elem_offset;
+    p.rope_theta = q.rope_theta; p.kv_capacity = q.kv_capacity;
+  }
 
   // lanes per row: narrow rows share a wave between several rows
   const int lpr = p.nchunks > 32 ? 64 : (p.nchunks > 16 ? 32 : 16);
@@ -295,7 +378,7 @@ hipError_t launch_gemv(const MatmulArgs& a, const Tune& t, hipStream_t s) {
   p.ntiles = (a.N + rpw - 1) / rpw;
 
   const uint32_t padded_chunks = (p.nchunks + 63u) & ~63u;
-  const size_t smem = (size_t)padded_chunks * 64 + (size_t)padded_chunks * 4;
+  const size_t smem = (size_t)padded_chunks * 64 + (size_t)padded_chunks * 4 + (a.qkv ? (size_t)(a.qkv->head_dim / 2) * 8 : 0);
 
   const uint32_t wg_tiles = (p.ntiles + waves - 1) / waves;
   gx = gx / pairs;
@@ -305,6 +388,10 @@ hipError_t launch_gemv(const MatmulArgs& a, const Tune& t, hipStream_t s) {
   const uint32_t threads = waves * 64;
 
   // dense M>1 handled by the caller looping rows; here one activation row
+  if (a.qkv) {
+    if (a.bits == 4) return a.affine ? launch_qkv<4, true>(p, lpr, grid, threads, smem, s) : launch_qkv<4, false>(p, lpr, grid, threads, smem, s);
+    return hipErrorInvalidValue;  // rejected by the entry point
+  }
   if (gated) {
     if (a.bits == 8) return hipErrorInvalidValue;  // rejected by the entry point
     if (a.bits == 4) return a.affine ? launch_gated<4, true>(p, lpr, grid, threads, smem, s) : launch_gated<4, false>(p, lpr, grid, threads, smem, s);

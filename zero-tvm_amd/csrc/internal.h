@@ -5,6 +5,18 @@
 
 namespace ztvm {
 
+// The fused QKV form (QKV matmul + RoPE + KV append): where the rotated pairs go.
+struct QkvArgs {
+  _Float16* q_out;
+  _Float16* kv_pages;
+  const int32_t* position_map;
+  uint32_t heads, kv_heads, head_dim;
+  uint32_t page_size, kv_page_stride, head_page_stride, v_page_offset;  // f16 elements
+  uint32_t position_map_elem_offset, pages_elem_offset;
+  uint64_t kv_capacity;
+  float rope_theta;
+};
+
 // Resolved launch arguments for every kernel family (device pointers typed).
 struct MatmulArgs {
   void* out;
@@ -17,6 +29,7 @@ struct MatmulArgs {
   const uint32_t* up_weights = nullptr;
   const _Float16* up_scales = nullptr;
   const _Float16* up_biases = nullptr;
+  const QkvArgs* qkv = nullptr;  // with qkv set, N counts rotary pairs and up_* is the same matrix half a head further
   uint32_t M, N, K, k_packed, spr;
   uint32_t bits, affine, out_f32;
   uint32_t slots, tokens;  // slots == 0: dense

@@ -375,6 +375,60 @@ int ztvm_ffn_gated(ztvm_ctx* ctx, const ztvm_matmul_desc* desc, uint64_t up_weig
   return ZTVM_OK;
 }
 
+int ztvm_qkv_fused(ztvm_ctx* ctx, const ztvm_qkv_fused_desc* d) {
+  if (!ctx) return fail(nullptr, ZTVM_E_INVALID, "null context");
+  if (!d) return fail(ctx, ZTVM_E_INVALID, "ztvm_qkv_fused: null descriptor");
+  if (d->bits != 4) return fail(ctx, ZTVM_E_UNSUPPORTED, "ztvm_qkv_fused: 4-bit rows only (got %u)", d->bits);
+  if (d->affine > 1) return fail(ctx, ZTVM_E_INVALID, "ztvm_qkv_fused: affine must be 0 or 1");
+  if (!d->heads || !d->kv_heads || !d->head_dim || (d->head_dim & 1u))
+    return fail(ctx, ZTVM_E_INVALID, "ztvm_qkv_fused: heads, kv_heads and an even head_dim are required");
+  if (d->head_dim > 512u) return fail(ctx, ZTVM_E_UNSUPPORTED, "ztvm_qkv_fused: head_dim %u > 512", d->head_dim);
+  if (!d->k_packed) return fail(ctx, ZTVM_E_INVALID, "ztvm_qkv_fused: K_PACKED must be > 0");
+  const uint64_t K = (uint64_t)d->k_packed * 8u;
+  const uint32_t G = d->affine ? 64u : 32u;
+  if (K % G || d->scales_per_row != K / G || K > (1u << 24))
+    return fail(ctx, ZTVM_E_INVALID, "ztvm_qkv_fused: SCALES_PER_ROW=%u does not match K=%llu at group %u", d->scales_per_row, (unsigned long long)K, G);
+  if (!d->page_size || !d->kv_page_stride || !d->head_page_stride)
+    return fail(ctx, ZTVM_E_INVALID, "ztvm_qkv_fused: page_size, kv_page_stride and head_page_stride must be > 0");
+  if ((uint64_t)d->page_size * d->head_dim > d->head_page_stride || (uint64_t)d->kv_heads * d->head_page_stride > d->v_page_offset ||
+      (uint64_t)d->v_page_offset + (uint64_t)d->kv_heads * d->head_page_stride > d->kv_page_stride)
+    return fail(ctx, ZTVM_E_INVALID, "ztvm_qkv_fused: page layout overlaps (page_size*head_dim <= head_page_stride, kv_heads*head_page_stride <= v_page_offset, v_page_offset + kv_heads*head_page_stride <= kv_page_stride)");
+  if (!(d->rope_theta > 0.f)) return fail(ctx, ZTVM_E_INVALID, "ztvm_qkv_fused: rope_theta must be > 0");
+  if (!d->q_out || !d->kv_pages || !d->hidden || !d->scales || !d->weights || !d->position_map)
+    return fail(ctx, ZTVM_E_INVALID, "ztvm_qkv_fused: null buffer");
+  if (d->affine && !d->biases) return fail(ctx, ZTVM_E_INVALID, "ztvm_qkv_fused: affine rows have no bias buffer");
+  if ((d->hidden | d->weights | d->scales | (d->affine ? d->biases : 0)) & 15u) return fail(ctx, ZTVM_E_INVALID, "ztvm_qkv_fused: hidden, weights, scales and biases must be 16-byte aligned");
+  if (((d->q_out | d->kv_pages) & 1u) || (d->position_map & 3u)) return fail(ctx, ZTVM_E_INVALID, "ztvm_qkv_fused: misaligned buffer");
+  const uint32_t half = d->head_dim / 2;
+  const uint64_t half_w = (uint64_t)half * d->k_packed * 4u, half_s = (uint64_t)half * d->scales_per_row * 2u;
+  if ((half_w | half_s) & 15u)
+    return fail(ctx, ZTVM_E_UNSUPPORTED, "ztvm_qkv_fused: half a head of rows (%u) must be a multiple of 16 bytes of weights and of scales", half);
+  QkvArgs q{};
+  q.q_out = reinterpret_cast<_Float16*>(d->q_out);
+  q.kv_pages = reinterpret_cast<_Float16*>(d->kv_pages);
+  q.position_map = reinterpret_cast<const int32_t*>(d->position_map);
+  q.heads = d->heads; q.kv_heads = d->kv_heads; q.head_dim = d->head_dim;
+  q.page_size = d->page_size; q.kv_page_stride = d->kv_page_stride; q.head_page_stride = d->head_page_stride;
+  q.v_page_offset = d->v_page_offset; q.position_map_elem_offset = d->position_map_elem_offset;
+  q.pages_elem_offset = d->pages_elem_offset; q.kv_capacity = d->kv_capacity; q.rope_theta = d->rope_theta;
+  MatmulArgs a{};
+  a.in = reinterpret_cast<const _Float16*>(d->hidden);
+  a.scales = reinterpret_cast<const _Float16*>(d->scales);
+  a.weights = reinterpret_cast<const uint32_t*>(d->weights);
+  a.biases = reinterpret_cast<const _Float16*>(d->biases);
+  a.out = q.q_out;
+  a.M = 1; a.N = (d->heads + 2u * d->kv_heads) * half;  // rotary pairs
+  a.K = (uint32_t)K; a.k_packed = d->k_packed; a.spr = d->scales_per_row;
+  a.bits = 4; a.affine = d->affine;
+  // the pair's second row lives half a head further in the same matrix
+  a.up_weights = a.weights + (size_t)half * d->k_packed;
+  a.up_scales = a.scales + (size_t)half * d->scales_per_row;
+  a.up_biases = d->affine ? a.biases + (size_t)half * d->scales_per_row : nullptr;
+  a.qkv = &q;
+  HIP_TRY(ctx, launch_gemv(a, ctx->tune, ctx->stream));
+  return ZTVM_OK;
+}
+
 int ztvm_dequant(ztvm_ctx* ctx, const ztvm_matmul_desc* desc) {
   if (!ctx) return fail(nullptr, ZTVM_E_INVALID, "null context");
   char why[256];

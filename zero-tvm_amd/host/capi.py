@@ -16,7 +16,7 @@ E_INVALID, E_HIP, E_UNSUPPORTED, E_NODEVICE = -1, -2, -3, -4
 EXPORTS = [
     "ztvm_abi_version", "ztvm_last_error", "ztvm_create", "ztvm_destroy", "ztvm_device_info",
     "ztvm_alloc", "ztvm_free", "ztvm_upload", "ztvm_download", "ztvm_fill", "ztvm_copy", "ztvm_sync",
-    "ztvm_matmul_validate", "ztvm_matmul_resolve", "ztvm_matmul", "ztvm_ffn_gated", "ztvm_dequant",
+    "ztvm_matmul_validate", "ztvm_matmul_resolve", "ztvm_matmul", "ztvm_ffn_gated", "ztvm_qkv_fused", "ztvm_dequant",
     "ztvm_record_begin", "ztvm_record_end", "ztvm_submit", "ztvm_cmdbuf_destroy",
     "ztvm_event_create", "ztvm_event_destroy", "ztvm_event_record", "ztvm_event_elapsed_ms",
     "ztvm_set_option", "ztvm_get_option",
@@ -39,6 +39,15 @@ class MatmulDesc(C.Structure):
         "bits", "affine", "out_f32", "kernel", "M", "N", "k_packed", "scales_per_row", "slots", "tokens",
         "in_slot_stride", "out_slot_stride", "in_tok_stride", "out_tok_stride", "ids_stride", "experts")] + [
         (n, C.c_uint64) for n in ("out", "in_", "scales", "weights", "biases", "ids")]
+
+
+class QkvFusedDesc(C.Structure):
+    """Mirror of ztvm_qkv_fused_desc."""
+    _fields_ = [(n, C.c_uint32) for n in (
+        "bits", "affine", "k_packed", "scales_per_row", "heads", "kv_heads", "head_dim", "page_size", "kv_page_stride",
+        "head_page_stride", "v_page_offset", "position_map_elem_offset", "pages_elem_offset")] + [
+        ("rope_theta", C.c_float), ("kv_capacity", C.c_uint64)] + [
+        (n, C.c_uint64) for n in ("q_out", "kv_pages", "hidden", "scales", "weights", "position_map", "biases")]
 
 
 _lib = None
@@ -81,6 +90,7 @@ def load():
     L.ztvm_get_option.argtypes = [vp, C.c_char_p, C.POINTER(C.c_int)]
     u32, u64 = C.c_uint32, C.c_uint64
     L.ztvm_ffn_gated.argtypes = [vp, C.POINTER(MatmulDesc), u64, u64, u64]
+    L.ztvm_qkv_fused.argtypes = [vp, C.POINTER(QkvFusedDesc)]
     L.ztvm_silu_mul.argtypes = [vp, u64, u64, u32, u32]
     L.ztvm_moe_combine.argtypes = [vp, u64, u64, u64, u32, u32, u32]
     L.ztvm_moe_router_logits.argtypes = [vp, u64, u64, u64, u64, u64, u32, u32, u32, u32]
@@ -174,6 +184,9 @@ class Context:
 
     def ffn_gated(self, desc, up_weights, up_scales, up_biases=0):
         self._chk(self._L.ztvm_ffn_gated(self._h, C.byref(desc), up_weights, up_scales, up_biases))
+
+    def qkv_fused(self, desc):
+        self._chk(self._L.ztvm_qkv_fused(self._h, C.byref(desc)))
 
     def dequant(self, desc):
         self._chk(self._L.ztvm_dequant(self._h, C.byref(desc)))

@@ -462,6 +462,58 @@ napi_value RepackDequantSplit(napi_env env, napi_callback_info info) {  // (ctx,
   return rc ? throw_ztvm(env, (ztvm_ctx*)p, rc, "ztvm_repack_dequant_split") : undefined(env);
 }
 
+napi_value QkvFused(napi_env env, napi_callback_info info) {  // (ctx, desc): keys are the ztvm_qkv_fused_desc field names
+  napi_value a[2];
+  void* p;
+  if (!get_args(env, info, 2, a) || !get_ptr(env, a[0], &p)) return nullptr;
+  ztvm_qkv_fused_desc d;
+  memset(&d, 0, sizeof d);
+  struct F32 { const char* name; uint32_t ztvm_qkv_fused_desc::*field; };
+  static const F32 u32s[] = {
+      {"bits", &ztvm_qkv_fused_desc::bits}, {"affine", &ztvm_qkv_fused_desc::affine}, {"k_packed", &ztvm_qkv_fused_desc::k_packed},
+      {"scales_per_row", &ztvm_qkv_fused_desc::scales_per_row}, {"heads", &ztvm_qkv_fused_desc::heads},
+      {"kv_heads", &ztvm_qkv_fused_desc::kv_heads}, {"head_dim", &ztvm_qkv_fused_desc::head_dim},
+      {"page_size", &ztvm_qkv_fused_desc::page_size}, {"kv_page_stride", &ztvm_qkv_fused_desc::kv_page_stride},
+      {"head_page_stride", &ztvm_qkv_fused_desc::head_page_stride}, {"v_page_offset", &ztvm_qkv_fused_desc::v_page_offset},
+      {"position_map_elem_offset", &ztvm_qkv_fused_desc::position_map_elem_offset},
+      {"pages_elem_offset", &ztvm_qkv_fused_desc::pages_elem_offset}};
+  for (const F32& f : u32s) {
+    napi_value v;
+    bool has = false;
+    napi_has_named_property(env, a[1], f.name, &has);
+    if (!has) continue;
+    napi_get_named_property(env, a[1], f.name, &v);
+    if (napi_get_value_uint32(env, v, &(d.*(f.field))) != napi_ok) {
+      napi_throw_type_error(env, nullptr, (std::string("ztvm addon: descriptor field '") + f.name + "' must be a number").c_str());
+      return nullptr;
+    }
+  }
+  struct F64 { const char* name; uint64_t ztvm_qkv_fused_desc::*field; };
+  static const F64 u64s[] = {{"kv_capacity", &ztvm_qkv_fused_desc::kv_capacity}, {"q_out", &ztvm_qkv_fused_desc::q_out},
+                             {"kv_pages", &ztvm_qkv_fused_desc::kv_pages}, {"hidden", &ztvm_qkv_fused_desc::hidden},
+                             {"scales", &ztvm_qkv_fused_desc::scales}, {"weights", &ztvm_qkv_fused_desc::weights},
+                             {"position_map", &ztvm_qkv_fused_desc::position_map}, {"biases", &ztvm_qkv_fused_desc::biases}};
+  for (const F64& f : u64s) {
+    napi_value v;
+    bool has = false;
+    napi_has_named_property(env, a[1], f.name, &has);
+    if (!has) continue;
+    napi_get_named_property(env, a[1], f.name, &v);
+    if (!get_u64(env, v, &(d.*(f.field)))) return nullptr;
+  }
+  napi_value v;
+  bool has = false;
+  napi_has_named_property(env, a[1], "rope_theta", &has);
+  if (has) {
+    double t = 0;
+    napi_get_named_property(env, a[1], "rope_theta", &v);
+    napi_get_value_double(env, v, &t);
+    d.rope_theta = (float)t;
+  }
+  int rc = ztvm_qkv_fused((ztvm_ctx*)p, &d);
+  return rc ? throw_ztvm(env, (ztvm_ctx*)p, rc, "ztvm_qkv_fused") : undefined(env);
+}
+
 napi_value Init(napi_env env, napi_value exports) {
   struct E { const char* name; napi_callback fn; };
   static const E table[] = {
@@ -471,7 +523,7 @@ napi_value Init(napi_env env, napi_value exports) {
       {"recordEnd", RecordEnd}, {"submit", Submit}, {"cmdbufDestroy", CmdbufDestroy}, {"setOption", SetOption},
       {"siluMul", SiluMul}, {"moeCombine", MoeCombine}, {"moeRouterLogits", MoeRouterLogits}, {"moeRouterTopk", MoeRouterTopk},
       {"moeSlotTranslate", MoeSlotTranslate}, {"ffnGated", FfnGated}, {"repackPart", RepackPart},
-      {"repackPermuteRows", RepackPermuteRows}, {"repackDequantSplit", RepackDequantSplit}};
+      {"repackPermuteRows", RepackPermuteRows}, {"repackDequantSplit", RepackDequantSplit}, {"qkvFused", QkvFused}};
   for (const E& e : table) {
     napi_value fn;
     if (napi_create_function(env, e.name, NAPI_AUTO_LENGTH, e.fn, nullptr, &fn) != napi_ok) return nullptr;

@@ -265,6 +265,24 @@ class Device {
     if (group.pipeline !== pipeline) throw new Error("ffnGated: bind group was built for '" + group.pipeline.label + "', not '" + pipeline.label + "'")
     addon().ffnGated(this.ctx, this.descriptor(group, wgX, wgY, wgZ), this._a(upWeights), this._a(upScales), this._a(upBiases))
   }
+  /**
+   * qkv_fused*.wgsl: bindings [q_out, kv_pages, hidden, scales, weights, position_map, (biases)], the PODArgs
+   * {position_map_elem_offset, pages_elem_offset} and the model constants of the shader prelude
+   * (heads, kvHeads, headDim, pageSize, kvPageStride, headPageStride, vPageOffset, ropeTheta).
+   */
+  qkvFused(bufs, pod, model) {
+    const w = pod.words, a = (b) => this._a(b)
+    const K = model.d
+    addon().qkvFused(this.ctx, {
+      bits: 4, affine: model.affine ? 1 : 0, k_packed: K / 8, scales_per_row: K / (model.affine ? 64 : 32),
+      heads: model.heads, kv_heads: model.kvHeads, head_dim: model.headDim, page_size: model.pageSize,
+      kv_page_stride: model.kvPageStride, head_page_stride: model.headPageStride, v_page_offset: model.vPageOffset,
+      position_map_elem_offset: w[0], pages_elem_offset: w[1], rope_theta: model.ropeTheta,
+      kv_capacity: BigInt(Math.floor(bufs[1].size / 2)),
+      q_out: a(bufs[0]), kv_pages: a(bufs[1]), hidden: a(bufs[2]), scales: a(bufs[3]), weights: a(bufs[4]),
+      position_map: a(bufs[5]), biases: bufs[6] ? a(bufs[6]) : 0n,
+    })
+  }
   beginEncoder() { addon().recordBegin(this.ctx) }
   finishEncoder() { return addon().recordEnd(this.ctx) }
   submit(cmdbuf) { addon().submit(this.ctx, cmdbuf) }
