@@ -274,6 +274,33 @@ def main():
         wb = synth.weight_bytes(6144, 4096)
         extra["qkv_fused_rope_kvappend_K4096_N6144"] = {"us": round(ms * 1e3, 3), "GB/s": round(wb / ms / 1e6, 1),
                                                         "hbm_frac": round(wb / ms / 1e6 / HBM_PEAK_GBS, 4)}
+        # the four weight-streaming dispatches of one 8B decoder layer with the fused forms: QKV + RoPE + KV append,
+        # o_proj, gate + up + SiLU, down (attention itself is not part of this path): 122.7 MB of weights per layer
+        lsets = []
+        for r in range(6):
+            o_b, _ = upload_set(ctx, synth, 4096, 4096, 4, salt=500 + r)
+            up_b, _ = upload_set(ctx, synth, 4096, 14336, 4, salt=520 + r)
+            hbuf = ctx.alloc(14336 * 2)
+            g0, d0 = sets[r % args.sets][0], sets[r % args.sets][1]
+            gated = capi.MatmulDesc(bits=4, affine=1, M=1, N=14336, k_packed=512, scales_per_row=64, out=hbuf, in_=g0.in_,
+                                    scales=g0.scales, weights=g0.weights, biases=g0.biases)
+            down = capi.MatmulDesc(bits=4, affine=1, M=1, N=4096, k_packed=1792, scales_per_row=224, out=d0.out, in_=hbuf,
+                                   scales=d0.scales, weights=d0.weights, biases=d0.biases)
+            lsets.append((qs[r % 8], make_desc(capi, 4, 4096, 4096, 1, o_b), gated, (up_b["w"], up_b["s"], up_b["b"]), down))
+
+        def layer(L):
+            q_, o_, g_, u_, d_ = L
+            ctx.qkv_fused(q_)
+            ctx.matmul(o_)
+            ctx.ffn_gated(g_, *u_)
+            ctx.matmul(d_)
+
+        layer(lsets[0])
+        ms = timed_graph(ctx, [lambda L=lsets[j % 6]: layer(L) for j in range(60)]) / 60
+        lbytes = (synth.weight_bytes(6144, 4096) + synth.weight_bytes(4096, 4096) + 2 * synth.weight_bytes(14336, 4096)
+                  + synth.weight_bytes(4096, 14336))
+        extra["decode_layer_8b_four_dispatches"] = {"us": round(ms * 1e3, 2), "GB/s": round(lbytes / ms / 1e6, 1),
+                                                    "hbm_frac": round(lbytes / ms / 1e6 / HBM_PEAK_GBS, 4), "weight_MB": round(lbytes / 1e6, 1)}
         # small batches through the weight-streaming kernel: int4 M in {8, 32, 128} and configs[4]'s int3 M=8
         for bits, M in ((4, 8), (4, 32), (4, 128), (3, 8)):
             src = gsets if bits == 4 else None

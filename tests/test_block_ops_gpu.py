@@ -319,3 +319,58 @@ def test_ffn_gated_rejects(ctx, capi):
         desc.kernel = capi.KERNEL_GEMM
         with pytest.raises(capi.ZtvmError):
             ctx.ffn_gated(desc, p, p, p)
+
+
+# ---------------------------------------------------------------- recorded replay ----------------------------
+
+def test_recorded_block_replays_match_eager(ctx, capi, synth, oracle):
+    """The whole routed FFN (five dispatches with the gated form) recorded into one command buffer and replayed
+    with new activations each time: every replay equals the eager result bit for bit, including the routing."""
+    D, F, E, K, tokens = 512, 256, 12, 3, 2
+    S = K + 1
+    _, rw, rs, _ = router_case(8, D, E + 1, tokens, 5)
+    rs = (rs.astype(np.float32) * 0.02).astype(np.float16)
+    rb = (-127.5 * rs.astype(np.float32)).astype(np.float16)
+    wg, wu, wd = (synth.packed_weights((E + 1) * F, D), synth.packed_weights((E + 1) * F, D, salt=2),
+                  synth.packed_weights((E + 1) * D, F, salt=3))
+    sg, su, sd = (synth.scales((E + 1) * F, D), synth.scales((E + 1) * F, D, salt=2), synth.scales((E + 1) * D, F, salt=3))
+    bg, bu, bd = synth.biases((E + 1) * F, D, sg), synth.biases((E + 1) * F, D, su, salt=2), synth.biases((E + 1) * D, F, sd, salt=3)
+    with Dev(ctx) as d:
+        X = d.empty(tokens * D * 2, fill=0)
+        logits, ids, score = d.empty(tokens * (E + 1) * 4, fill=0), d.empty(tokens * S * 4, fill=0), d.empty(tokens * S * 4, fill=0)
+        h, down, y = d.empty(tokens * S * F * 2, fill=0), d.empty(tokens * S * D * 2, fill=0), d.empty(tokens * D * 2, fill=0)
+        RW, RS, RB = d.put(rw), d.put(rs), d.put(rb)
+        WG, SG, BG, WU, SU, BU, WD, SD, BD = (d.put(a) for a in (wg, sg, bg, wu, su, bu, wd, sd, bd))
+        common = dict(bits=4, affine=1, M=1, slots=S, tokens=tokens, ids=ids, ids_stride=S, experts=E + 1)
+        gate = capi.MatmulDesc(N=F, k_packed=D // 8, scales_per_row=D // 64, in_slot_stride=0, in_tok_stride=D, out_slot_stride=F,
+                               out_tok_stride=S * F, out=h, in_=X, weights=WG, scales=SG, biases=BG, **common)
+        dn = capi.MatmulDesc(N=D, k_packed=F // 8, scales_per_row=F // 64, in_slot_stride=F, in_tok_stride=S * F,
+                             out_slot_stride=D, out_tok_stride=S * D, out=down, in_=h, weights=WD, scales=SD, biases=BD, **common)
+
+        def block():
+            ctx.moe_router_logits(logits, X, RW, RS, RB, 8, D, E + 1, tokens)
+            ctx.moe_router_topk(ids, score, logits, E, K, True, True, tokens)
+            ctx.ffn_gated(gate, WU, SU, BU)
+            ctx.matmul(dn)
+            ctx.moe_combine(y, down, score, tokens, D, S)
+
+        ctx.record_begin()
+        block()
+        cb = ctx.record_end()
+        try:
+            seen = set()
+            for rep in range(4):
+                x = synth.activations(tokens, D, salt=40 + rep)
+                ctx.upload(X, x)
+                block()
+                eager = (ctx.download(y, tokens * D * 2, np.uint16), ctx.download(ids, tokens * S * 4, np.uint32))
+                ctx.fill(y, 0, tokens * D * 2)
+                ctx.fill(ids, 0xFF, tokens * S * 4)
+                ctx.submit(cb)
+                replay = (ctx.download(y, tokens * D * 2, np.uint16), ctx.download(ids, tokens * S * 4, np.uint32))
+                assert np.array_equal(eager[0], replay[0]) and np.array_equal(eager[1], replay[1]), rep
+                assert eager[0].any()
+                seen.add(eager[1].tobytes())
+            assert len(seen) > 1, "different activations route differently"
+        finally:
+            ctx.cmdbuf_destroy(cb)
