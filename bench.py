@@ -84,7 +84,9 @@ def verify(ctx, oracle, capi, desc, host, bits, K, N, M, f16w=False):
     ctx.matmul(desc)
     y = ctx.download(desc.out, M * N * 2, np.float16).astype(np.float64).reshape(M, N)
     rows = min(M, 4)
-    mode = oracle.MODE_F16W if f16w else oracle.MODE_FORMULA_F32
+    # byte-valued weights give outputs near 100: an f32-accumulated reference carries more noise of its own than the
+    # 1e-2 bar leaves at outputs near zero, so those rows are checked against the f64 formula
+    mode = oracle.MODE_F16W if f16w else (oracle.MODE_FORMULA_F64 if bits == 8 else oracle.MODE_FORMULA_F32)
     ref = oracle.gemm(mode, bits, True, rows, N, K, x[:rows], w, s, b, threads=oracle.max_threads())
     err = float(np.max(np.abs(y[:rows] - ref) / (np.abs(ref) + 1e-2)))
     if not np.all(np.isfinite(y)) or err >= 1e-2:
@@ -301,16 +303,15 @@ def main():
                   + synth.weight_bytes(4096, 14336))
         extra["decode_layer_8b_four_dispatches"] = {"us": round(ms * 1e3, 2), "GB/s": round(lbytes / ms / 1e6, 1),
                                                     "hbm_frac": round(lbytes / ms / 1e6 / HBM_PEAK_GBS, 4), "weight_MB": round(lbytes / 1e6, 1)}
-        # small batches through the weight-streaming kernel: int4 M in {8, 32, 128} and configs[4]'s int3 M=8
-        for bits, M in ((4, 8), (4, 32), (4, 128), (3, 8)):
-            src = gsets if bits == 4 else None
+        # small batches through the weight-streaming kernel: int4 M in {8, 32, 128}, configs[4]'s int3 M=8, 8-bit M in {8, 128}
+        for bits, M in ((4, 8), (4, 32), (4, 128), (3, 8), (8, 8), (8, 128)):
             if bits == 4:
                 descs = [make_desc(capi, 4, 4096, 14336, M, b) for b, _ in gsets]
                 host0 = gsets[0][1]
             else:
-                i3m = [upload_set(ctx, synth, 4096, 14336, 3, salt=300 + r, M=M) for r in range(3)]
-                descs = [make_desc(capi, 3, 4096, 14336, M, b) for b, _ in i3m]
-                host0 = i3m[0][1]
+                other = [upload_set(ctx, synth, 4096, 14336, bits, salt=300 + 10 * bits + r, M=M) for r in range(3)]
+                descs = [make_desc(capi, bits, 4096, 14336, M, b) for b, _ in other]
+                host0 = other[0][1]
             verify(ctx, oracle, capi, descs[0], host0, bits, 4096, 14336, M)
             ms = timed_graph(ctx, [lambda d=descs[j % 3]: ctx.matmul(d) for j in range(36)]) / 36
             wb = synth.weight_bytes(14336, 4096, bits=bits)

@@ -100,7 +100,7 @@ def test_rules_and_routing(capi):
                          weights=4096, biases=4096)
     assert capi.validate(ok)[0] == 0 and capi.resolve(ok) == capi.KERNEL_GEMV
     ok.M = 300
-    assert capi.resolve(ok) == capi.KERNEL_GEMV          # no 8-bit form of the other families: one pass per row
+    assert capi.resolve(ok) == capi.KERNEL_SKINNY        # the weight-streaming kernel at any M; no 8-bit tile GEMM
     ok.kernel = capi.KERNEL_GEMM
     assert capi.validate(ok)[0] == capi.E_UNSUPPORTED
     sym = capi.MatmulDesc(bits=8, affine=0, M=1, N=64, k_packed=256, scales_per_row=32, out=4096, in_=4096, scales=4096, weights=4096)

@@ -1,9 +1,10 @@
-"""GPU parity of the weight-streaming matrix-core kernel (family 'skinny', 2 <= M <= 128 rows by
+"""GPU parity of the weight-streaming matrix-core kernel (family 'skinny', 17 <= M <= 128 rows by
 default, any M when asked for).
 
 The cases mirror the reference's small-batch checks (tests/kernels/compile-qwen35.mjs:963-1152:
 M=6 N=64, M=31 N=256, M=47 N=200 at K=2560; scripts/gemm-sweep-native.mjs:374: 13x96x128) and add
-the formats the reference ships for the same dispatch: symmetric group-32 and the 3-bit stream.
+the formats the reference ships for the same dispatch: symmetric group-32, the 3-bit stream and the
+8-bit affine layout (src/compiler/shaders/int8_affine_batched.wgsl).
 Bars: |y-ref|/(|ref|+1e-2) < 1e-2 against the from-the-formula f64 oracle (the kernel multiplies
 exact integer weights and scales in f32, so it holds the GEMV's bar), rows past M untouched,
 results independent of M and of the tile height, one-hot rows bit-exact.
@@ -35,7 +36,7 @@ def make(synth, bits, affine, CAP, N, K, regime="A"):
     return A, w, s, b
 
 
-FORMATS = [(4, True), (4, False), (3, True)]
+FORMATS = [(4, True), (4, False), (3, True), (8, True)]
 CASES = [(2, 8, 64, 2560), (6, 8, 64, 2560), (31, 64, 256, 2560), (33, 64, 256, 2560), (47, 64, 200, 2560), (13, 64, 96, 128),
          (64, 64, 136, 64), (65, 128, 136, 192), (100, 128, 264, 1024), (128, 128, 128, 512), (130, 256, 136, 512),
          (300, 320, 264, 1024)]
@@ -73,7 +74,9 @@ def test_k_split(ctx, capi, synth, oracle, bits, affine, ksplit):
         ctx.set_option("skinny.ksplit", 0)
     ref = oracle.gemm(oracle.MODE_FORMULA_F64, bits, affine, M, N, K, A, w, s, b, threads=8)
     assert rel_err(got.view(np.float16).astype(np.float64), ref, 1e-2) < 1e-2
-    assert rel_err(got32.view(np.float32).astype(np.float64), ref, 1.0) < 1e-5
+    # f32 accumulation noise; byte-valued weights make the per-group integer sums 16 times larger than nibbles do,
+    # and the products that cancel in the total are rounded at that size
+    assert rel_err(got32.view(np.float32).astype(np.float64), ref, 1.0) < (4e-5 if bits == 8 else 1e-5)
 
 
 def test_one_hot_pins_streamed_weights(ctx, capi, synth, oracle):
@@ -110,10 +113,14 @@ def test_config5_int3_m8(ctx, capi, synth, oracle):
 
 
 def test_auto_picks_skinny(capi):
-    for M, want in ((1, capi.KERNEL_GEMV), (2, capi.KERNEL_SKINNY), (128, capi.KERNEL_SKINNY), (129, capi.KERNEL_GEMM)):
+    for M, want in ((1, capi.KERNEL_GEMV), (17, capi.KERNEL_SKINNY), (128, capi.KERNEL_SKINNY), (129, capi.KERNEL_GEMM)):
         desc = capi.MatmulDesc(bits=4, affine=1, M=M, N=256, k_packed=64, scales_per_row=8, out=4096, in_=4096, scales=4096,
                                weights=4096, biases=4096)
         assert capi.resolve(desc) == want, M
     desc = capi.MatmulDesc(bits=3, affine=1, M=300, N=256, k_packed=48, scales_per_row=8, out=4096, in_=4096, scales=4096,
                            weights=4096, biases=4096)
     assert capi.resolve(desc) == capi.KERNEL_SKINNY  # the tile GEMM has no 3-bit path
+    for M in (20, 300):
+        desc = capi.MatmulDesc(bits=8, affine=1, M=M, N=256, k_packed=128, scales_per_row=8, out=4096, in_=4096, scales=4096,
+                               weights=4096, biases=4096)
+        assert capi.resolve(desc) == capi.KERNEL_SKINNY  # nor an 8-bit one

@@ -47,6 +47,8 @@ struct Tune {
   int i8_wg_per_cu = 0;
   int skinny_wg_per_cu = 0;
   int skinny_ksplit = 0;     // workgroups sharing the k range of one skinny tile (0: chosen from M, N, K)
+  int rows_wg_per_cu = 0;    // the row-group GEMV: workgroups per CU and waves per workgroup (0: chosen from the LDS it stages)
+  int rows_waves = 0;
   int gemm_tile = 0;        // 0 auto
   int gemm_xcd_swizzle = 1;
 };
@@ -79,6 +81,12 @@ hipError_t launch_dequant_split(void* out, const void* w, const void* scales, co
                                 uint32_t nope, uint32_t v, uint32_t* counter, hipStream_t s);
 
 bool skinny_supports(const MatmulArgs& a);
+// the row-group GEMV (gemv_rows.hip), 1 <= M <= 16
+bool rows_supports(const MatmulArgs& a);
+size_t rows_scratch_bytes(const MatmulArgs& a);
+hipError_t launch_rows(const MatmulArgs& a, const Tune& t, void* scratch, hipStream_t s);
+// out[i] = sum over the k splits of partial[k][i], in split order; count a multiple of four (skinny.hip)
+hipError_t launch_reduce_partials(const float* partial, void* out, uint32_t count, uint32_t ksplit, bool out_f32, hipStream_t s);
 bool gemm_supports(const MatmulArgs& a);
 
 }  // namespace ztvm

@@ -1,5 +1,5 @@
 // Weight-streaming matrix-core kernel for 2 <= M rows of activations:
-//   Y[m,n] = sum_k A[m,k] * w[n,k],  w = s*q + b (4-bit or 3-bit, group 64) or s*(q-7) (4-bit, group 32).
+//   Y[m,n] = sum_k A[m,k] * w[n,k],  w = s*q + b (4-bit, 3-bit or 8-bit, group 64) or s*(q-7) (4-bit, group 32).
 //
 // Replaces the reference's small-batch generators (src/compiler/shaders/int4_matmul.gen.ts:
 // int4MatmulBatchedWGSL :430-540, int4MatmulBatchedDynWGSL :580-695, int4MatmulTiledMWGSL
@@ -23,7 +23,9 @@
 // The unpackers produce eight values in slot order [v0,v4,v1,v5,v2,v6,v3,v7]; a pre-pass writes
 // a copy of the activations with every 8-element chunk in that order (and the group sums), so
 // the 12-instruction natural-order unpack becomes 9 (4-bit) and the 3-bit stream unpacks with
-// funnel shifts only.
+// funnel shifts only. 8-bit words unpack to the pairs (v0,v2), (v1,v3), so for that format the copy
+// is in the order [v0,v2,v1,v3,v4,v6,v5,v7] (src/compiler/shaders/int8_affine_batched.wgsl is the
+// reference's kernel for it: K_PACKED = K/4, four values per word).
 #include "internal.h"
 #include "mma.h"
 
@@ -51,7 +53,7 @@ struct StreamParams {
 // One thread per 16-byte chunk, eight consecutive lanes = one 64-k group, summed across lanes.
 __global__ __launch_bounds__(256) void prep_kernel(const _Float16* __restrict__ in, _Float16* __restrict__ inp,
                                                    _Float16* __restrict__ xs16, uint32_t M, uint32_t K, uint32_t xs_stride,
-                                                   uint32_t want_xs) {
+                                                   uint32_t want_xs, uint32_t order8) {
   const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
   const uint32_t cpr = K / 8, total = M * cpr, G = K / 64;
   if (want_xs) {
@@ -66,7 +68,7 @@ __global__ __launch_bounds__(256) void prep_kernel(const _Float16* __restrict__ 
 #pragma unroll
   for (int i = 0; i < 8; i++) {
     s += (float)v[i];
-    w[slot_of(i)] = v[i];
+    w[i] = order8 ? v[value_in_slot8(i)] : v[value_in_slot(i)];
   }
   *reinterpret_cast<h8*>(inp + (size_t)m * K + (size_t)c * 8) = w;
   if (want_xs) {
@@ -86,8 +88,8 @@ typedef uint32_t u32x3_a4 __attribute__((ext_vector_type(3), aligned(4)));
 
 // Registers of one step's weights of a lane.
 struct WRegs {
-  u32x4 a;     // 4-bit: words 4h..4h+3 (affine) or 0..3 (symmetric)
-  u32x4 b;     // 4-bit symmetric: words 4..7
+  u32x4 a;     // 4-bit: words 4h..4h+3 (affine) or 0..3 (symmetric); 8-bit: words 8h..8h+3
+  u32x4 b;     // 4-bit symmetric: words 4..7; 8-bit: words 8h+4..8h+7
   u32x3 c;     // 3-bit: words 3h..3h+2
   uint32_t s;  // one f16 scale (affine) or two (symmetric)
 };
@@ -103,14 +105,14 @@ constexpr int DEPTH = 4;
 
 template <int MB, int BITS, bool AFFINE, bool CLAMP>
 __global__ __launch_bounds__(64 * WAVES) void stream_kernel(const StreamParams p) {
-  static_assert(BITS == 4 || (BITS == 3 && AFFINE), "formats");
+  static_assert(BITS == 4 || ((BITS == 3 || BITS == 8) && AFFINE), "formats");
   static_assert(DEPTH % 2 == 0, "the LDS buffer of a step is its position in the unrolled group, mod 2");
   constexpr int ROWS = MB * 32;
   constexpr uint32_t STAGE_BYTES = ROWS * 128;
   constexpr int RPB = AFFINE ? 1 : 2;  // runs = groups per block and step
   constexpr int NRUN = MB * RPB;
   constexpr int MPR = 4 / RPB;         // MFMAs per run
-  constexpr int W_STEP_WORDS = BITS == 4 ? 8 : 6;
+  constexpr int W_STEP_WORDS = BITS == 4 ? 8 : (BITS == 8 ? 16 : 6);
 
   extern __shared__ __align__(16) unsigned char smem[];
 
@@ -168,7 +170,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_kernel(const StreamParams p
   };
 
   // ---- weights and scales of this lane's column
-  const uint32_t* w_src = p.weights + (size_t)n * p.row_words + (size_t)s_begin * W_STEP_WORDS + (BITS == 3 ? h * 3 : (AFFINE ? h * 4 : 0));
+  const uint32_t* w_src = p.weights + (size_t)n * p.row_words + (size_t)s_begin * W_STEP_WORDS + (BITS == 3 ? h * 3 : (BITS == 8 ? h * 8 : (AFFINE ? h * 4 : 0)));
   const _Float16* sc_src = p.scales + (size_t)n * p.spr + (size_t)s_begin * RPB;
   auto fetch_w = [&](WRegs& r) __attribute__((always_inline)) {
     if constexpr (BITS == 3) {
@@ -176,7 +178,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_kernel(const StreamParams p
       r.c = (u32x3){v.x, v.y, v.z};
     } else {
       r.a = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(w_src));
-      if constexpr (!AFFINE) r.b = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(w_src + 4));
+      if constexpr (!AFFINE || BITS == 8) r.b = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(w_src + 4));
     }
     if constexpr (AFFINE) r.s = *reinterpret_cast<const uint16_t*>(sc_src);
     else r.s = *reinterpret_cast<const uint32_t*>(sc_src);
@@ -189,7 +191,10 @@ __global__ __launch_bounds__(64 * WAVES) void stream_kernel(const StreamParams p
   // B operand t: eight exact integers (q, or q-7) in slot order
   auto unpack_t = [&](const WRegs& r, int t) __attribute__((always_inline)) {
     h2 q[4];
-    if constexpr (BITS == 4) {
+    if constexpr (BITS == 8) {
+      unpack8_word(t < 2 ? r.a[2 * t] : r.b[2 * t - 4], q, uc);
+      unpack8_word(t < 2 ? r.a[2 * t + 1] : r.b[2 * t - 3], q + 2, uc);
+    } else if constexpr (BITS == 4) {
       uint32_t w;
       if constexpr (AFFINE) {
         w = r.a[t];
@@ -276,13 +281,6 @@ __global__ __launch_bounds__(64 * WAVES) void stream_kernel(const StreamParams p
   part[0] = zero;
   part[1] = zero;
 
-  static_for<DEPTH>([&](auto jc) {
-    constexpr int j = decltype(jc)::value;
-    if (j < nsteps) {
-      fetch_w(wq[j]);
-      fetch_a(aq[j], a_src);
-    }
-  });
 
   // one step: position j in the ring; REFILL: the ring slot is refilled for step s+DEPTH
   auto step = [&](auto jc, auto refill_c) __attribute__((always_inline)) {
@@ -328,9 +326,27 @@ __global__ __launch_bounds__(64 * WAVES) void stream_kernel(const StreamParams p
   };
   using yes = std::integral_constant<bool, true>;
   using no = std::integral_constant<bool, false>;
-  // groups of DEPTH steps whose refills are all in range: no branches, exact wait counts
+  // groups of DEPTH steps whose refills are all in range: no branches, exact wait counts. The ring is
+  // primed on a path of its own: a wait count is fixed per instruction, so the loop's waits can only be
+  // as loose as the tightest path that reaches the loop, and a priming sequence with a branch per slot
+  // (short k ranges) would have every wait in the loop drain all loads in flight.
   uint32_t s = 0;
-  for (; s + 2 * DEPTH <= nsteps; s += DEPTH) static_for<DEPTH>([&](auto jc) { step(jc, yes{}); });
+  if (nsteps >= 2 * DEPTH) {
+    static_for<DEPTH>([&](auto jc) {
+      constexpr int j = decltype(jc)::value;
+      fetch_w(wq[j]);
+      fetch_a(aq[j], a_src);
+    });
+    for (; s + 2 * DEPTH <= nsteps; s += DEPTH) static_for<DEPTH>([&](auto jc) { step(jc, yes{}); });
+  } else {
+    static_for<DEPTH>([&](auto jc) {
+      constexpr int j = decltype(jc)::value;
+      if (j < nsteps) {
+        fetch_w(wq[j]);
+        fetch_a(aq[j], a_src);
+      }
+    });
+  }
   // up to 2*DEPTH - 1 remaining steps
   for (; s < nsteps; s += DEPTH) {
     static_for<DEPTH>([&](auto jc) {
@@ -420,9 +436,14 @@ size_t align256(size_t v) { return (v + 255) / 256 * 256; }
 }  // namespace
 
 // Dense, K a multiple of 64, byte offsets within 32 bits.
+hipError_t launch_reduce_partials(const float* partial, void* out, uint32_t count, uint32_t ksplit, bool out_f32, hipStream_t s) {
+  hipLaunchKernelGGL(reduce_kernel, dim3((count / 4 + 255) / 256), dim3(256), 0, s, partial, out, count, ksplit, (uint32_t)out_f32);
+  return hipGetLastError();
+}
+
 bool skinny_supports(const MatmulArgs& a) {
   if (a.slots != 0 || a.K % KS != 0 || a.M < 1) return false;
-  if (!(a.bits == 4 || (a.bits == 3 && a.affine))) return false;
+  if (!(a.bits == 4 || ((a.bits == 3 || a.bits == 8) && a.affine))) return false;
   const uint64_t lim = 1ull << 32;
   return (uint64_t)a.M * a.K * 2 < lim && (uint64_t)a.M * (xs_stride_of(a) + 1) * 2 < lim;
 }
@@ -458,17 +479,17 @@ hipError_t launch_skinny(const MatmulArgs& a, const Tune& t, void* scratch, hipS
   {
     const uint32_t pad = a.affine ? p.xs_stride - 2 * (a.K / 64) : 0, cpr = a.K / 8;
     const uint32_t nthr = a.M * (cpr > pad ? cpr : pad);  // one thread per chunk, and enough for the padding columns
-    hipLaunchKernelGGL(prep_kernel, dim3((nthr + 255) / 256), dim3(256), 0, s, a.in, inp, xs16, a.M, a.K, p.xs_stride, (uint32_t)a.affine);
+    hipLaunchKernelGGL(prep_kernel, dim3((nthr + 255) / 256), dim3(256), 0, s, a.in, inp, xs16, a.M, a.K, p.xs_stride, (uint32_t)a.affine,
+                       (uint32_t)(a.bits == 8));
   }
   hipError_t e;
   if (a.bits == 3) e = launch_fmt<3, true>(p, mb, s);
+  else if (a.bits == 8) e = launch_fmt<8, true>(p, mb, s);
   else if (a.affine) e = launch_fmt<4, true>(p, mb, s);
   else e = launch_fmt<4, false>(p, mb, s);
   if (e != hipSuccess) return e;
   if (p.ksplit > 1) {
-    const uint32_t count = a.M * a.N;  // N % 4 == 0 whenever ksplit > 1
-    hipLaunchKernelGGL(reduce_kernel, dim3((count / 4 + 255) / 256), dim3(256), 0, s, p.partial, a.out, count, p.ksplit, (uint32_t)a.out_f32);
-    return hipGetLastError();
+    return launch_reduce_partials(p.partial, a.out, a.M * a.N, p.ksplit, a.out_f32 != 0, s);  // N % 4 == 0 whenever ksplit > 1
   }
   return hipSuccess;
 }

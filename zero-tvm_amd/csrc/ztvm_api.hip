@@ -68,7 +68,7 @@ int validate(const ztvm_matmul_desc* d, char* why, size_t n, bool need_in_out) {
   if (d->bits == 3 && !d->affine) { why_set(why, n, "q3 requires affine (3-bit ships only in the MLX-affine layout)"); return ZTVM_E_INVALID; }
   if (d->bits == 8 && !d->affine) { why_set(why, n, "8-bit requires affine (8-bit ships only in the MLX-affine layout)"); return ZTVM_E_INVALID; }
   if (d->slots && !d->affine) { why_set(why, n, "moe requires affine (the MoE weights are MLX affine-quantised)"); return ZTVM_E_INVALID; }
-  if (d->kernel > ZTVM_KERNEL_GEMM) { why_set(why, n, "unknown kernel family %u", d->kernel); return ZTVM_E_INVALID; }
+  if (d->kernel > ZTVM_KERNEL_ROWS) { why_set(why, n, "unknown kernel family %u", d->kernel); return ZTVM_E_INVALID; }
   if (!d->N) { why_set(why, n, "N must be > 0"); return ZTVM_E_INVALID; }
   if (!d->k_packed) { why_set(why, n, "K_PACKED must be > 0"); return ZTVM_E_INVALID; }
   const uint64_t kbits = (uint64_t)d->k_packed * 32u;
@@ -132,6 +132,7 @@ int resolve(const MatmulArgs& a, uint32_t want, char* why, size_t n) {
   const bool moe = a.slots > 0;
   const bool sk = !moe && skinny_supports(a);
   const bool ge = !moe && gemm_supports(a);
+  const bool ro = !moe && rows_supports(a);
   if (want == ZTVM_KERNEL_GEMV) return ZTVM_KERNEL_GEMV;
   if (want == ZTVM_KERNEL_SKINNY) {
     if (!sk) { why_set(why, n, "kernel: asked for 'skinny', which cannot run this dispatch (moe=%d, M=%u)", (int)moe, a.M); return ZTVM_E_UNSUPPORTED; }
@@ -141,7 +142,12 @@ int resolve(const MatmulArgs& a, uint32_t want, char* why, size_t n) {
     if (!ge) { why_set(why, n, "kernel: asked for 'gemm', which cannot run this dispatch (moe=%d, bits=%u, out_f32=%u, K=%u)", (int)moe, a.bits, a.out_f32, a.K); return ZTVM_E_UNSUPPORTED; }
     return ZTVM_KERNEL_GEMM;
   }
+  if (want == ZTVM_KERNEL_ROWS) {
+    if (!ro) { why_set(why, n, "kernel: asked for 'rows', which cannot run this dispatch (moe=%d, M=%u, K=%u, N=%u)", (int)moe, a.M, a.K, a.N); return ZTVM_E_UNSUPPORTED; }
+    return ZTVM_KERNEL_ROWS;
+  }
   if (moe || a.M == 1) return ZTVM_KERNEL_GEMV;
+  if (ro) return ZTVM_KERNEL_ROWS;
   if (ge && a.M > 128) return ZTVM_KERNEL_GEMM;
   if (sk) return ZTVM_KERNEL_SKINNY;
   if (ge) return ZTVM_KERNEL_GEMM;
@@ -162,6 +168,8 @@ const Option kOptions[] = {
     {"i8.wg_per_cu", &Tune::i8_wg_per_cu},
     {"skinny.wg_per_cu", &Tune::skinny_wg_per_cu},
     {"skinny.ksplit", &Tune::skinny_ksplit},
+    {"rows.wg_per_cu", &Tune::rows_wg_per_cu},
+    {"rows.waves", &Tune::rows_waves},
     {"gemm.tile", &Tune::gemm_tile},
     {"gemm.xcd_swizzle", &Tune::gemm_xcd_swizzle},
 };
@@ -303,9 +311,10 @@ int ztvm_matmul(ztvm_ctx* ctx, const ztvm_matmul_desc* desc) {
   const int fam = resolve(a, desc->kernel, why, sizeof why);
   if (fam < 0) return fail(ctx, fam, "ztvm_matmul: %s", why);
   switch (fam) {
+    case ZTVM_KERNEL_ROWS:
     case ZTVM_KERNEL_SKINNY:
     case ZTVM_KERNEL_GEMM: {
-      const size_t need = fam == ZTVM_KERNEL_GEMM ? gemm_scratch_bytes(a) : skinny_scratch_bytes(a, ctx->tune);
+      const size_t need = fam == ZTVM_KERNEL_GEMM ? gemm_scratch_bytes(a) : (fam == ZTVM_KERNEL_ROWS ? rows_scratch_bytes(a) : skinny_scratch_bytes(a, ctx->tune));
       if (need > ctx->scratch_bytes) {
         // growing means a free + malloc, which a command buffer cannot hold
         if (ctx->recording)
@@ -318,6 +327,7 @@ int ztvm_matmul(ztvm_ctx* ctx, const ztvm_matmul_desc* desc) {
         ctx->scratch_bytes = need;
       }
       if (fam == ZTVM_KERNEL_GEMM) HIP_TRY(ctx, launch_gemm(a, ctx->tune, ctx->scratch, ctx->stream));
+      else if (fam == ZTVM_KERNEL_ROWS) HIP_TRY(ctx, launch_rows(a, ctx->tune, ctx->scratch, ctx->stream));
       else HIP_TRY(ctx, launch_skinny(a, ctx->tune, ctx->scratch, ctx->stream));
       break;
     }

@@ -9,8 +9,8 @@ import os
 _PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB_PATH = os.path.join(_PKG, "lib", "libztvm_hip.so")
 
-KERNEL_AUTO, KERNEL_GEMV, KERNEL_SKINNY, KERNEL_GEMM = 0, 1, 2, 3
-KERNEL_NAMES = {0: "auto", 1: "gemv", 2: "skinny", 3: "gemm"}
+KERNEL_AUTO, KERNEL_GEMV, KERNEL_SKINNY, KERNEL_GEMM, KERNEL_ROWS = 0, 1, 2, 3, 4
+KERNEL_NAMES = {0: "auto", 1: "gemv", 2: "skinny", 3: "gemm", 4: "rows"}
 E_INVALID, E_HIP, E_UNSUPPORTED, E_NODEVICE = -1, -2, -3, -4
 
 EXPORTS = [

@@ -46,7 +46,7 @@ export declare class Device {
   submit(cmdbuf: unknown): void
   sync(): void
 }
-export declare const KERNEL: { AUTO: 0; GEMV: 1; SKINNY: 2; GEMM: 3 }
+export declare const KERNEL: { AUTO: 0; GEMV: 1; SKINNY: 2; GEMM: 3; ROWS: 4 }
 export declare const INT4_MATMUL_VARIANTS: ReadonlyArray<Int4MatmulOpts>
 export declare const GEMM_ENTRIES: ReadonlyArray<string>
 export declare const INT8_ENTRIES: ReadonlyArray<string>

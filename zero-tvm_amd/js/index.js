@@ -22,7 +22,7 @@ function addon() {
   return native
 }
 
-const KERNEL = { AUTO: 0, GEMV: 1, SKINNY: 2, GEMM: 3 }
+const KERNEL = { AUTO: 0, GEMV: 1, SKINNY: 2, GEMM: 3, ROWS: 4 }
 
 // ---- variant naming ----------------------------------------------------------------------------
 
