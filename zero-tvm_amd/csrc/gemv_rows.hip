@@ -29,6 +29,8 @@ namespace ztvm {
 namespace {
 
 constexpr int PASS = 16;              // chunks per wave pass = blocks of the 4x4x4 instruction
+constexpr int UNROLL = 2;             // passes per pipeline stage: two loads per lane go out together
+constexpr int STEP = PASS * UNROLL;   // chunks per stage; staged k ranges are padded to whole stages
 constexpr uint32_t LDS_ROW_BUDGET = 72 * 1024 / 8;  // bytes of LDS a staged activation row may take (8 rows: 72 KB)
 
 struct RowsParams {
@@ -45,8 +47,8 @@ typedef uint32_t words3 __attribute__((ext_vector_type(3), aligned(4)));
 
 template <int WORDS>
 struct RowFrag {
-  uint32_t w[WORDS];
-  _Float16 s, b;
+  uint32_t w[UNROLL][WORDS];
+  _Float16 s[UNROLL], b[UNROLL];
 };
 
 template <int CTRL>
@@ -68,8 +70,8 @@ __global__ __launch_bounds__(1024) void rows_kernel(const RowsParams p) {
   // this workgroup's chunks of every row
   const uint32_t c_begin = blockIdx.y * p.cps;
   const uint32_t c_count = p.nchunks - c_begin < p.cps ? p.nchunks - c_begin : p.cps;
-  const uint32_t npasses = (c_count + PASS - 1) / PASS;
-  const uint32_t cpad = npasses * PASS;
+  const uint32_t npasses = (c_count + STEP - 1) / STEP;  // pipeline stages per row tile
+  const uint32_t cpad = npasses * STEP;
 
   // LDS: 16-byte pieces of x at ((group*4 + piece)*cpad + chunk)*4 + row%4, so the 64 lanes of a
   // read touch 64 consecutive pieces; then float sums at [chunk][row]
@@ -80,27 +82,30 @@ __global__ __launch_bounds__(1024) void rows_kernel(const RowsParams p) {
   kc.init();
 
   auto issue = [&](RowFrag<FW>& f, uint32_t tile, uint32_t pass) {
-    uint32_t cl = pass * PASS + b;
-    cl = cl < c_count ? cl : c_count - 1;  // a clamped chunk meets staged zeros
-    const uint32_t c = c_begin + cl;
     uint32_t row = tile * 4 + j;
-    row = row < p.N ? row : p.N - 1;       // a clamped row is never stored
-    const uint32_t g = AFFINE ? (c >> 1) : c;
-    const uint32_t* wp = p.weights + (size_t)row * p.k_packed + (size_t)c * WPC;
-    if (BITS == 8) {
-      const u32x4 v0 = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp));
-      const u32x4 v1 = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp) + 1);
-      f.w[0] = v0.x; f.w[1] = v0.y; f.w[2] = v0.z; f.w[3] = v0.w;
-      f.w[4 % FW] = v1.x; f.w[5 % FW] = v1.y; f.w[6 % FW] = v1.z; f.w[7 % FW] = v1.w;
-    } else if (BITS == 4) {
-      const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp));
-      f.w[0] = v.x; f.w[1] = v.y; f.w[2] = v.z; f.w[3] = v.w;
-    } else {
-      const words3 v = __builtin_nontemporal_load(reinterpret_cast<const words3*>(wp));
-      f.w[0] = v.x; f.w[1] = v.y; f.w[2] = v.z; f.w[3] = 0;
+    row = row < p.N ? row : p.N - 1;  // a clamped row is never stored
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+      uint32_t cl = pass * STEP + u * PASS + b;
+      cl = cl < c_count ? cl : c_count - 1;  // a clamped chunk meets staged zeros
+      const uint32_t c = c_begin + cl;
+      const uint32_t g = AFFINE ? (c >> 1) : c;
+      const uint32_t* wp = p.weights + (size_t)row * p.k_packed + (size_t)c * WPC;
+      if (BITS == 8) {
+        const u32x4 v0 = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp));
+        const u32x4 v1 = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp) + 1);
+        f.w[u][0] = v0.x; f.w[u][1] = v0.y; f.w[u][2] = v0.z; f.w[u][3] = v0.w;
+        f.w[u][4 % FW] = v1.x; f.w[u][5 % FW] = v1.y; f.w[u][6 % FW] = v1.z; f.w[u][7 % FW] = v1.w;
+      } else if (BITS == 4) {
+        const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp));
+        f.w[u][0] = v.x; f.w[u][1] = v.y; f.w[u][2] = v.z; f.w[u][3] = v.w;
+      } else {
+        const words3 v = __builtin_nontemporal_load(reinterpret_cast<const words3*>(wp));
+        f.w[u][0] = v.x; f.w[u][1] = v.y; f.w[u][2] = v.z; f.w[u][3] = 0;
+      }
+      f.s[u] = p.scales[(size_t)row * p.spr + g];
+      if (AFFINE) f.b[u] = p.biases[(size_t)row * p.spr + g];
     }
-    f.s = p.scales[(size_t)row * p.spr + g];
-    if (AFFINE) f.b = p.biases[(size_t)row * p.spr + g];
   };
 
   const uint32_t wave_stride = gridDim.x * waves;
@@ -109,24 +114,43 @@ __global__ __launch_bounds__(1024) void rows_kernel(const RowsParams p) {
   RowFrag<FW> fa, fb;
   issue(fa, have ? tile : p.ntiles - 1, 0);  // the weight stream starts while x is staged
 
-  // ---- stage x: one (row, chunk) per thread and turn
-  for (uint32_t idx = tid; idx < (uint32_t)M4 * cpad; idx += blockDim.x) {
-    const uint32_t m = idx / cpad, cl = idx - m * cpad;
-    const bool real = m < p.M && cl < c_count;
-    float s = 0.f;
+  // ---- stage x: one (row, chunk) per thread and turn, two turns in flight. Only the M real rows are
+  // staged: row i of a 4x4x4 product depends on row i of A alone, so what the unused rows of a
+  // group hold (anything) stays in sums that are never stored.
+  {
+    const uint32_t pairs = p.M * cpad;
+    auto place = [&](uint32_t idx, const h8 (&v)[4], bool real) __attribute__((always_inline)) {
+      const uint32_t m = idx / cpad, cl = idx - m * cpad;
+      float s = 0.f;
 #pragma unroll
-    for (int piece = 0; piece < 4; piece++) {
-      h8 o = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (real) {
-        const h8 v = reinterpret_cast<const h8*>(p.in + (size_t)m * p.K + (size_t)(c_begin + cl) * 32u)[piece];
+      for (int piece = 0; piece < 4; piece++) {
+        h8 o;
 #pragma unroll
-        for (int sl = 0; sl < 8; sl++) o[sl] = v[BITS == 8 ? value_in_slot8(sl) : value_in_slot(sl)];
+        for (int sl = 0; sl < 8; sl++) o[sl] = real ? v[piece][BITS == 8 ? value_in_slot8(sl) : value_in_slot(sl)] : (_Float16)0.f;
 #pragma unroll
-        for (int i = 0; i < 8; i++) s += (float)v[i];
+        for (int i = 0; i < 8; i++) s += (float)v[piece][i];
+        x_pieces[(((m >> 2) * 4 + piece) * cpad + cl) * 4 + (m & 3u)] = o;
       }
-      x_pieces[(((m >> 2) * 4 + piece) * cpad + cl) * 4 + (m & 3u)] = o;
+      xsum[cl * M4 + m] = real ? s : 0.f;
+    };
+    auto fetch = [&](uint32_t idx, h8 (&v)[4]) __attribute__((always_inline)) {
+      // chunks past the end of the range (padding of the last pass) read the row's last real chunk and are staged as zeros
+      const uint32_t m = idx / cpad, cl = idx - m * cpad;
+      const uint32_t cc = cl < c_count ? cl : c_count - 1;
+      const h8* src = reinterpret_cast<const h8*>(p.in + (size_t)m * p.K + (size_t)(c_begin + cc) * 32u);
+#pragma unroll
+      for (int piece = 0; piece < 4; piece++) v[piece] = src[piece];
+      return cl < c_count;
+    };
+    for (uint32_t idx = tid; idx < pairs; idx += 2 * blockDim.x) {
+      h8 v0[4], v1[4];
+      const uint32_t idx1 = idx + blockDim.x;
+      const bool two = idx1 < pairs;
+      const bool r0 = fetch(idx, v0);
+      const bool r1 = fetch(two ? idx1 : idx, v1);
+      place(idx, v0, r0);
+      if (two) place(idx1, v1, r1);
     }
-    xsum[cl * M4 + m] = s;
   }
   __syncthreads();
 
@@ -152,42 +176,45 @@ __global__ __launch_bounds__(1024) void rows_kernel(const RowsParams p) {
     // always issued (past the end: the last tile again, never consumed): loads under a branch would
     // make every wait below drain the loads just issued as well
     issue(nxt, nhave ? ntile : p.ntiles - 1, npass);
-    const uint32_t cl = pass * PASS + b;
     XGroup xa, xb;
-    read_x(xa, cl, 0);
+    read_x(xa, pass * STEP + b, 0);
     __builtin_amdgcn_sched_barrier(0);  // loads and LDS reads first; the unpack below covers their latency
 
-    h2 q[16];
-    if constexpr (BITS == 8) unpack8_chunk(cur.w, q, kc);
-    else if constexpr (BITS == 4) unpack4_chunk(cur.w[0], cur.w[1], cur.w[2], cur.w[3], q, kc);
-    else unpack3_chunk(cur.w[0], cur.w[1], cur.w[2], q, kc);
-    const float s = (float)cur.s;
-    const float bias = AFFINE ? (float)cur.b : 0.f;
-    auto group = [&](const XGroup& x, int mg) __attribute__((always_inline)) {
-      f4 d0 = {0.f, 0.f, 0.f, 0.f}, d1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int w = 0; w < 4; w++) {
-        const h8 xv = x.v[w];
-        const h4 xlo = {xv[0], xv[1], xv[2], xv[3]}, xhi = {xv[4], xv[5], xv[6], xv[7]};
-        const h4 qlo = {q[4 * w].x, q[4 * w].y, q[4 * w + 1].x, q[4 * w + 1].y};
-        const h4 qhi = {q[4 * w + 2].x, q[4 * w + 2].y, q[4 * w + 3].x, q[4 * w + 3].y};
-        d0 = __builtin_amdgcn_mfma_f32_4x4x4f16(xlo, qlo, d0, 0, 0, 0);
-        d1 = __builtin_amdgcn_mfma_f32_4x4x4f16(xhi, qhi, d1, 0, 0, 0);
-      }
+    for (int u = 0; u < UNROLL; u++) {
+      const uint32_t cl = pass * STEP + u * PASS + b;
+      h2 q[16];
+      if constexpr (BITS == 8) unpack8_chunk(cur.w[u], q, kc);
+      else if constexpr (BITS == 4) unpack4_chunk(cur.w[u][0], cur.w[u][1], cur.w[u][2], cur.w[u][3], q, kc);
+      else unpack3_chunk(cur.w[u][0], cur.w[u][1], cur.w[u][2], q, kc);
+      const float s = (float)cur.s[u];
+      const float bias = AFFINE ? (float)cur.b[u] : 0.f;
+      auto group = [&](const XGroup& x, int mg) __attribute__((always_inline)) {
+        f4 d0 = {0.f, 0.f, 0.f, 0.f}, d1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int i = 0; i < 4; i++) {
-        const float dot = d0[i] + d1[i];
-        acc[mg * 4 + i] += AFFINE ? __builtin_fmaf(s, dot, bias * x.sum[i]) : s * __builtin_fmaf(-7.f, x.sum[i], dot);
-      }
-    };
-    // groups alternate between two register sets: the next group's pieces are read while this one multiplies
+        for (int w = 0; w < 4; w++) {
+          const h8 xv = x.v[w];
+          const h4 xlo = {xv[0], xv[1], xv[2], xv[3]}, xhi = {xv[4], xv[5], xv[6], xv[7]};
+          const h4 qlo = {q[4 * w].x, q[4 * w].y, q[4 * w + 1].x, q[4 * w + 1].y};
+          const h4 qhi = {q[4 * w + 2].x, q[4 * w + 2].y, q[4 * w + 3].x, q[4 * w + 3].y};
+          d0 = __builtin_amdgcn_mfma_f32_4x4x4f16(xlo, qlo, d0, 0, 0, 0);
+          d1 = __builtin_amdgcn_mfma_f32_4x4x4f16(xhi, qhi, d1, 0, 0, 0);
+        }
 #pragma unroll
-    for (int mg = 0; mg < MG; mg += 2) {
-      if (mg + 1 < MG) read_x(xb, cl, mg + 1);
-      group(xa, mg);
-      if (mg + 1 < MG) {
-        if (mg + 2 < MG) read_x(xa, cl, mg + 2);
-        group(xb, mg + 1);
+        for (int i = 0; i < 4; i++) {
+          const float dot = d0[i] + d1[i];
+          acc[mg * 4 + i] += AFFINE ? __builtin_fmaf(s, dot, bias * x.sum[i]) : s * __builtin_fmaf(-7.f, x.sum[i], dot);
+        }
+      };
+      // groups alternate between two register sets: the next pieces (the next group's, or the next
+      // chunk's first group) are read while this group multiplies
+#pragma unroll
+      for (int mg = 0; mg < MG; mg++) {
+        XGroup& now = (u * MG + mg) % 2 ? xb : xa;
+        XGroup& then = (u * MG + mg) % 2 ? xa : xb;
+        if (mg + 1 < MG) read_x(then, cl, mg + 1);
+        else if (u + 1 < UNROLL) read_x(then, cl + PASS, 0);
+        group(now, mg);
       }
     }
 
@@ -227,9 +254,9 @@ __global__ __launch_bounds__(1024) void rows_kernel(const RowsParams p) {
 }
 
 uint32_t chunks_per_split(uint32_t nchunks) {
-  const uint32_t most = LDS_ROW_BUDGET / 68u / PASS * PASS;  // 68 bytes of LDS per staged chunk and row
+  const uint32_t most = LDS_ROW_BUDGET / 68u / STEP * STEP;  // 68 bytes of LDS per staged chunk and row
   const uint32_t ksplit = (nchunks + most - 1) / most;
-  return ((nchunks + ksplit - 1) / ksplit + PASS - 1) / PASS * PASS;
+  return ((nchunks + ksplit - 1) / ksplit + STEP - 1) / STEP * STEP;
 }
 
 template <int BITS, bool AFFINE>
@@ -276,7 +303,7 @@ hipError_t launch_rows(const MatmulArgs& a, const Tune& t, void* scratch, hipStr
   p.ntiles = (a.N + 3) / 4;
   p.out_f32 = a.out_f32;
   const int mg = (int)(a.M + 3) / 4;
-  const size_t smem = (size_t)mg * 4 * p.cps * 68;  // cps is a whole number of passes
+  const size_t smem = (size_t)mg * 4 * p.cps * 68;  // cps is a whole number of stages
 
   // workgroups: as many as LDS holds per CU (at most three); one large workgroup where the staged
   // activations are big, so that they are staged once per CU
