@@ -48,8 +48,6 @@ struct GemvParams {
   uint32_t slots, in_slot_stride, out_slot_stride, in_tok_stride, out_tok_stride, ids_stride, experts;
 };
 
-// Three words of a 3-bit chunk: 12 bytes at a 4-byte aligned address.
-typedef uint32_t words3 __attribute__((ext_vector_type(3), aligned(4)));
 
 // LDS layout of x for chunk c: piece j (8 halves, 16 bytes) sits at 16-byte
 // slot (c/64)*256 + j*64 + c%64, so the 64 lanes of one ds_read_b128 touch 64
@@ -132,33 +130,49 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(const GemvParams p) {
   UnpackConsts kc;
   kc.init();
 
-  // Loads of one (tile, pass). Rows past N and chunks past K are clamped to a
-  // valid address (their contribution is masked later), so no lane diverges.
+  // Loads of one (tile, pass), as buffer loads: a uniform descriptor (this expert's matrix) plus one
+  // 32-bit byte offset per lane, and an offset past the end of the array returns zeros without
+  // touching memory. Rows past N are past the end by themselves (so are whole tiles past the last
+  // one: the pipeline fetches ahead without asking whether anything is left); chunks past K are
+  // sent there. No lane diverges, nothing is fetched twice and no load sits under a branch.
+  constexpr uint32_t NOWHERE = 0x80000000u;  // every matrix is shorter than this (checked by the entry points)
+  const uint32_t wbytes = QKV ? 0x7FFFFFFFu : p.N * p.k_packed * 4u, sbytes = QKV ? 0x7FFFFFFFu : p.N * p.spr * 2u;
+  const __amdgpu_buffer_rsrc_t wres = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(wbase), 0, wbytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t sres = __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16*>(sbase), 0, sbytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t bres = __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16*>(AFFINE ? bbase : sbase), 0, sbytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t wres2 = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(GATED ? wbase2 : wbase), 0, wbytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t sres2 = __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16*>(GATED ? sbase2 : sbase), 0, sbytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t bres2 = __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16*>(GATED && AFFINE ? bbase2 : sbase), 0, sbytes, 0x00020000);
   auto issue = [&](Frag<FR, FW>& f, uint32_t tile, uint32_t pass) {
     const uint32_t c = pass * LPR + lk;
-    const uint32_t cc = c < p.nchunks ? c : p.nchunks - 1;
-    const uint32_t g = AFFINE ? (cc >> 1) : cc;
+    const bool in_k = c < p.nchunks;
+    const uint32_t g = AFFINE ? (c >> 1) : c;
 #pragma unroll
     for (int r = 0; r < FR; r++) {
       const bool up = GATED && r >= ROWS;
       uint32_t rr = tile * RPW + (r % ROWS) * SUB + sub;
-      rr = rr < p.N ? rr : p.N - 1;
-      if (QKV) rr = qkv_pair(p, rr).row_lo;
-      const uint32_t* wp = (up ? wbase2 : wbase) + (size_t)rr * p.k_packed + (size_t)cc * WPC;
+      bool ok = in_k;
+      if (QKV) {  // pairs map to rows of the fused matrix, whose length the pair count does not give
+        ok = ok && rr < p.N;
+        rr = qkv_pair(p, rr < p.N ? rr : p.N - 1).row_lo;
+      }
+      const uint32_t woff = ok ? (rr * p.k_packed + c * WPC) * 4u : NOWHERE;
+      const uint32_t soff = ok ? (rr * p.spr + g) * 2u : NOWHERE;
+      const __amdgpu_buffer_rsrc_t wr = up ? wres2 : wres;
       if (BITS == 8) {
-        const u32x4 v0 = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp));
-        const u32x4 v1 = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp) + 1);
+        const u32x4 v0 = __builtin_amdgcn_raw_buffer_load_b128(wr, woff, 0, 2);  // 2: non-temporal
+        const u32x4 v1 = __builtin_amdgcn_raw_buffer_load_b128(wr, woff + 16, 0, 2);
         f.w[r][0] = v0.x; f.w[r][1] = v0.y; f.w[r][2] = v0.z; f.w[r][3] = v0.w;
         f.w[r][4 % FW] = v1.x; f.w[r][5 % FW] = v1.y; f.w[r][6 % FW] = v1.z; f.w[r][7 % FW] = v1.w;
       } else if (BITS == 4) {
-        const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp));
+        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(wr, woff, 0, 2);
         f.w[r][0] = v.x; f.w[r][1] = v.y; f.w[r][2] = v.z; f.w[r][3] = v.w;
       } else {
-        const words3 v = __builtin_nontemporal_load(reinterpret_cast<const words3*>(wp));
+        const u32x3 v = __builtin_amdgcn_raw_buffer_load_b96(wr, woff, 0, 2);
         f.w[r][0] = v.x; f.w[r][1] = v.y; f.w[r][2] = v.z; f.w[r][3] = 0;
       }
-      f.s[r] = (up ? sbase2 : sbase)[(size_t)rr * p.spr + g];
-      if (AFFINE) f.b[r] = (up ? bbase2 : bbase)[(size_t)rr * p.spr + g];
+      f.s[r] = __builtin_bit_cast(_Float16, __builtin_amdgcn_raw_buffer_load_b16(up ? sres2 : sres, soff, 0, 0));
+      if (AFFINE) f.b[r] = __builtin_bit_cast(_Float16, __builtin_amdgcn_raw_buffer_load_b16(up ? bres2 : bres, soff, 0, 0));
     }
   };
 
@@ -168,7 +182,7 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(const GemvParams p) {
   uint32_t tile = blockIdx.x * waves + wave, pass = 0;
   bool have = tile < p.ntiles;
   Frag<FR, FW> fa, fb;
-  if (have) issue(fa, tile, 0);
+  issue(fa, tile, 0);
 
   // ---- stage x: each thread converts whole chunks -------------------------
   h8* xs_pieces = reinterpret_cast<h8*>(smem);
@@ -211,7 +225,7 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(const GemvParams p) {
     uint32_t ntile = tile, npass = pass + 1;
     if (npass == p.npasses) { npass = 0; ntile += wave_stride; }
     const bool nhave = ntile < p.ntiles;
-    if (nhave) issue(nxt, ntile, npass);
+    issue(nxt, ntile, npass);  // past the last tile this fetches nothing
     // keep the loads above where they are: the scheduler would otherwise sink
     // the small scale/bias loads down to their first use
     __builtin_amdgcn_sched_barrier(0);

@@ -81,6 +81,8 @@ int validate(const ztvm_matmul_desc* d, char* why, size_t n, bool need_in_out) {
     why_set(why, n, "SCALES_PER_ROW=%u but K/group = %llu (K=%llu, group %u)", d->scales_per_row, (unsigned long long)(K / G), (unsigned long long)K, G);
     return ZTVM_E_INVALID;
   }
+  // the streaming kernels address a matrix with 32-bit byte offsets from its base
+  if ((uint64_t)d->N * d->k_packed * 4u >= (1ull << 31)) { why_set(why, n, "one weight matrix must stay under 2 GiB (N=%u rows of %u words)", d->N, d->k_packed); return ZTVM_E_INVALID; }
   if (need_in_out) {
     if (d->slots) {
       if (d->M != 1) { why_set(why, n, "moe dispatches one activation row per (token,slot): M must be 1 (got %u)", d->M); return ZTVM_E_INVALID; }
@@ -398,6 +400,8 @@ int ztvm_qkv_fused(ztvm_ctx* ctx, const ztvm_qkv_fused_desc* d) {
   const uint32_t G = d->affine ? 64u : 32u;
   if (K % G || d->scales_per_row != K / G || K > (1u << 24))
     return fail(ctx, ZTVM_E_INVALID, "ztvm_qkv_fused: SCALES_PER_ROW=%u does not match K=%llu at group %u", d->scales_per_row, (unsigned long long)K, G);
+  if ((uint64_t)(d->heads + 2u * d->kv_heads) * d->head_dim * d->k_packed * 4u >= (1ull << 31))
+    return fail(ctx, ZTVM_E_INVALID, "ztvm_qkv_fused: the fused weight matrix must stay under 2 GiB");
   if (!d->page_size || !d->kv_page_stride || !d->head_page_stride)
     return fail(ctx, ZTVM_E_INVALID, "ztvm_qkv_fused: page_size, kv_page_stride and head_page_stride must be > 0");
   if ((uint64_t)d->page_size * d->head_dim > d->head_page_stride || (uint64_t)d->kv_heads * d->head_page_stride > d->v_page_offset ||
