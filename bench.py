@@ -303,8 +303,9 @@ def main():
                   + synth.weight_bytes(4096, 14336))
         extra["decode_layer_8b_four_dispatches"] = {"us": round(ms * 1e3, 2), "GB/s": round(lbytes / ms / 1e6, 1),
                                                     "hbm_frac": round(lbytes / ms / 1e6 / HBM_PEAK_GBS, 4), "weight_MB": round(lbytes / 1e6, 1)}
-        # small batches through the weight-streaming kernel: int4 M in {8, 32, 128}, configs[4]'s int3 M=8, 8-bit M in {8, 128}
-        for bits, M in ((4, 8), (4, 32), (4, 128), (3, 8), (8, 8), (8, 128)):
+        # small batches: the row-group GEMV (M <= 16) and the weight-streaming matrix-core kernel (M <= 128); int4,
+        # configs[4]'s int3 M=8, and 8-bit rows
+        for bits, M in ((4, 2), (4, 4), (4, 8), (4, 16), (4, 32), (4, 128), (3, 8), (8, 8), (8, 128)):
             if bits == 4:
                 descs = [make_desc(capi, 4, 4096, 14336, M, b) for b, _ in gsets]
                 host0 = gsets[0][1]
@@ -315,7 +316,7 @@ def main():
             verify(ctx, oracle, capi, descs[0], host0, bits, 4096, 14336, M)
             ms = timed_graph(ctx, [lambda d=descs[j % 3]: ctx.matmul(d) for j in range(36)]) / 36
             wb = synth.weight_bytes(14336, 4096, bits=bits)
-            extra["skinny_int%d_M%d_K4096_N14336" % (bits, M)] = {
+            extra["batch_int%d_M%d_K4096_N14336" % (bits, M)] = {
                 "us": round(ms * 1e3, 2), "TFLOP/s": round(2.0 * M * 4096 * 14336 / ms / 1e9, 1),
                 "weights_GB/s": round(wb / ms / 1e6, 1), "family": capi.KERNEL_NAMES[capi.resolve(descs[0])]}
         # MoE expert block (configs[3]): 256 experts, top-8, hidden 2048, intermediate 512; gate + up + down per token batch

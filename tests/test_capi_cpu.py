@@ -73,6 +73,7 @@ def test_validator_accepts_reference_shapes(capi):
     (dict(slots=8, tokens=2, ids=0x6000, ids_stride=8, in_slot_stride=4, out_slot_stride=64), "multiples of 8"),
     (dict(slots=8, tokens=2, ids=0x6000, ids_stride=8, out_slot_stride=8), "overlap"),
     (dict(kernel=9), "kernel"),
+    (dict(N=1 << 20), "2 GiB"),                            # 2^20 rows of 512 words = 2 GiB: 32-bit byte offsets end here
 ])
 def test_validator_rejects(capi, kw, needle):
     rc, why = capi.validate(good(capi, **kw))
@@ -87,6 +88,17 @@ def test_explicit_kernel_that_cannot_run_is_an_error(capi):
     assert rc == capi.E_UNSUPPORTED and "asked for" in why
     with pytest.raises(capi.ZtvmError):
         capi.resolve(moe)
+
+
+def test_auto_picks_a_family_by_rows(capi):
+    """M = 1: per-row GEMV; 2..16: row-group GEMV; 17..128: weight-streaming matrix-core kernel; above: tile GEMM."""
+    for M, want in ((1, capi.KERNEL_GEMV), (2, capi.KERNEL_ROWS), (16, capi.KERNEL_ROWS), (17, capi.KERNEL_SKINNY),
+                    (128, capi.KERNEL_SKINNY), (129, capi.KERNEL_GEMM)):
+        assert capi.resolve(good(capi, M=M)) == want, M
+    assert capi.resolve(good(capi, M=8, bits=3, k_packed=384, scales_per_row=64)) == capi.KERNEL_ROWS
+    assert capi.resolve(good(capi, M=300, bits=3, k_packed=384, scales_per_row=64)) == capi.KERNEL_SKINNY
+    rc, why = capi.validate(good(capi, M=17, kernel=capi.KERNEL_ROWS))
+    assert rc == capi.E_UNSUPPORTED and "rows" in why
 
 
 def test_no_device_is_a_loud_error(capi):
