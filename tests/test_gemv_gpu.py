@@ -107,3 +107,32 @@ def test_int3_config5_m1(ctx, capi, synth, oracle):
     b = synth.biases(N, K, s)
     y = run_dense(ctx, capi, 3, True, 1, N, K, x, w, s, b)
     print("int3 rel err:", check(y, oracle, 3, True, 1, N, K, x, w, s, b))
+
+
+def test_seeded_random_shapes(ctx, capi, synth, oracle):
+    """Forty seeded GEMV shapes across the formats: ragged N, K from one scale group up, dense and f32 output."""
+    rng = np.random.default_rng(977)
+    formats = [(4, True), (4, False), (3, True), (8, True)]
+    for case in range(40):
+        bits, affine = formats[case % 4]
+        group = 64 if affine else 32
+        N = int(rng.integers(1, 400))
+        K = group * int(rng.choice([1, 2, 3, 7, 8, 16, 31, 64, 100, 224]))
+        out_f32 = int(case % 5 == 0)
+        x = synth.activations(1, K)
+        w = synth.packed_weights(N, K, bits=bits)
+        s = synth.scales(N, K, affine=affine)
+        b = synth.biases(N, K, s, "A") if affine else None
+        esz = 4 if out_f32 else 2
+        with Dev(ctx) as d:
+            out = d.empty(N * esz + 16, fill=0)
+            desc = capi.MatmulDesc(bits=bits, affine=int(affine), out_f32=out_f32, M=1, N=N, k_packed=K * bits // 32,
+                                   scales_per_row=K // group, out=out, in_=d.put(x), scales=d.put(s), weights=d.put(w),
+                                   biases=d.put(b) if affine else 0)
+            ctx.matmul(desc)
+            raw = ctx.download(out, N * esz + 16, np.uint8)
+        y = raw[:N * esz].view(np.float32 if out_f32 else np.float16).astype(np.float64)
+        ref = oracle.gemm(oracle.MODE_FORMULA_F64, bits, affine, 1, N, K, x, w, s, b, threads=8)[0]
+        err = rel_err(y, ref, 1e-2)
+        assert err < 1e-2, (case, bits, affine, N, K, err)
+        assert not raw[N * esz:].any(), "wrote past N"

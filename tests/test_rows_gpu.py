@@ -126,3 +126,21 @@ def test_auto_routing(capi):
                            weights=4096, biases=4096, kernel=capi.KERNEL_ROWS)
     with pytest.raises(capi.ZtvmError, match="rows"):
         capi.resolve(desc)
+
+
+def test_seeded_random_shapes(ctx, capi, synth, oracle):
+    """Forty seeded shapes across the formats: ragged N, K from one scale group to several k ranges, every M."""
+    rng = np.random.default_rng(20240607)
+    for case in range(40):
+        bits, affine = FORMATS[case % len(FORMATS)]
+        group = 64 if affine else 32
+        M = int(rng.integers(1, 17))
+        N = int(rng.integers(1, 300))
+        K = group * int(rng.choice([1, 2, 3, 5, 8, 17, 40, 64, 65, 100, 130]))
+        if K > 4096 and N % 4:
+            N += 4 - N % 4          # a split k range needs groups of four outputs
+        A, w, s, b = make(synth, bits, affine, M, N, K)
+        got = run(ctx, capi, bits, affine, M, M, N, K, A, w, s, b)
+        ref = oracle.gemm(oracle.MODE_FORMULA_F64, bits, affine, M, N, K, A, w, s, b, threads=8)
+        err = rel_err(got.view(np.float16).astype(np.float64), ref, 1e-2)
+        assert err < 1e-2, (case, bits, affine, M, N, K, err)
