@@ -276,6 +276,25 @@ def main():
         wb = synth.weight_bytes(6144, 4096)
         extra["qkv_fused_rope_kvappend_K4096_N6144"] = {"us": round(ms * 1e3, 3), "GB/s": round(wb / ms / 1e6, 1),
                                                         "hbm_frac": round(wb / ms / 1e6 / HBM_PEAK_GBS, 4)}
+        # the int8-KV pair at the same shape: QKV + RoPE to scratch rows, then the quantizer into the int8 pages
+        kslot, vslot = ctx.alloc(1024 * 2), ctx.alloc(1024 * 2)
+        i8pages, i8scales = ctx.alloc(64 * 8 * 16 * 2 * 32 * 4), ctx.alloc(64 * 8 * 16 * 2 * 2)
+        kvq = capi.KvQuantizeDesc(kv_heads=8, head_dim=128, page_size=16, tokens=1, pages_capacity_words=64 * 8 * 16 * 2 * 32,
+                                  scales_capacity=64 * 8 * 16 * 2, k_slot=kslot, v_slot=vslot, pages_i8=i8pages, scales=i8scales,
+                                  position_map=pmap)
+
+        def int8_pair(d):
+            ctx.qkv_fused_scratch(d, kslot, vslot)
+            ctx.kv_quantize_int8(kvq)
+
+        int8_pair(qs[0])
+        got_sc = ctx.download(i8scales, 64 * 8 * 16 * 2 * 2, np.float16).reshape(64, 8, 16, 2)[517 // 16, :, 517 % 16, :]
+        krow = np.abs(ctx.download(kslot, 1024 * 2, np.float16).astype(np.float32)).reshape(8, 128).max(axis=1) / np.float32(127)
+        if not np.array_equal(got_sc[:, 0], krow.astype(np.float16)):
+            raise SystemExit("bench: int8 KV scale check failed")
+        ms2 = timed_graph(ctx, [lambda d=qs[j % 8]: int8_pair(d) for j in range(160)]) / 160
+        ms1 = timed_graph(ctx, [lambda: ctx.kv_quantize_int8(kvq) for j in range(160)]) / 160
+        extra["qkv_scratch_then_kv_quantize_int8_K4096_N6144"] = {"us": round(ms2 * 1e3, 3), "kv_quantize_us": round(ms1 * 1e3, 3)}
         # the four weight-streaming dispatches of one 8B decoder layer with the fused forms: QKV + RoPE + KV append,
         # o_proj, gate + up + SiLU, down (attention itself is not part of this path): 122.7 MB of weights per layer
         lsets = []

@@ -194,6 +194,30 @@ typedef struct ztvm_qkv_fused_desc {
 } ztvm_qkv_fused_desc;
 ZTVM_API int ztvm_qkv_fused(ztvm_ctx* ctx, const ztvm_qkv_fused_desc* desc);
 
+/* The int8-KV-mode variant (src/compiler/shaders/qkv_fused_scratch.wgsl:14-150; engine-core.ts:849):
+ * the same math, but K (rotated) and V go to two f16 scratch rows k_slot / v_slot of
+ * kv_heads*head_dim elements each (row-major head, dim) instead of the paged cache; a
+ * ztvm_kv_quantize_int8 dispatch then writes the int8 cache. The descriptor's kv_pages, page
+ * layout and kv_capacity fields are not read. */
+ZTVM_API int ztvm_qkv_fused_scratch(ztvm_ctx* ctx, const ztvm_qkv_fused_desc* desc, uint64_t k_slot, uint64_t v_slot);
+
+/* kv_quantize_int8 (src/compiler/shaders/kv_quantize_int8.wgsl:47-164): per (token, kv head, side)
+ * one scale = max|x| / 127 (at least 1e-8) over the head's head_dim values, stored as f16, and
+ * q = clamp(round-half-even(x / scale), -127, 127) packed four to a u32 word. k_slot / v_slot are
+ * [tokens][kv_heads*head_dim] f16. Words: page . head . slot . side(K, V) . dim/4, i.e.
+ *   page_no*kv_heads*page_size*2*(head_dim/4) + head*page_size*2*(head_dim/4) + slot*2*(head_dim/4) + side*(head_dim/4) + dim/4 + pages_word_offset
+ * scales: page_no*kv_heads*page_size*2 + head*page_size*2 + slot*2 + side + scales_elem_offset,
+ * with (page_no, slot) from position_map[position_map_elem_offset + token]. tokens = grid y of the
+ * reference (1 on the decode path). A negative position, or an index at or past a capacity
+ * (0 = unchecked), writes nothing, so a bad position cannot fault the GPU. */
+typedef struct ztvm_kv_quantize_desc {
+  uint32_t kv_heads, head_dim, page_size, tokens;
+  uint32_t position_map_elem_offset, pages_word_offset, scales_elem_offset, reserved;
+  uint64_t pages_capacity_words, scales_capacity;
+  uint64_t k_slot, v_slot, pages_i8, scales, position_map;
+} ztvm_kv_quantize_desc;
+ZTVM_API int ztvm_kv_quantize_int8(ztvm_ctx* ctx, const ztvm_kv_quantize_desc* desc);
+
 /* Dequantize a weight stack to [N,K] f16 (out_f32=0) or f32 (out_f32=1):
  * w = fl32(q*s + b) (or (q-7)*s), f16 = RNE of that. Uses bits, affine, N,
  * k_packed, scales_per_row, weights, scales, biases and out of `desc`.

@@ -67,6 +67,8 @@ def lib():
         L.zo_slot_translate.restype, L.zo_slot_translate.argtypes = None, [u32p, u32p, C.c_uint32, u32p]
         L.zo_qkv_fused.restype = None
         L.zo_qkv_fused.argtypes = [C.c_uint32] * 10 + [C.c_double, C.c_int32, u16p, u32p, u16p, u16p, u16p, u16p]
+        L.zo_kv_quantize_int8.restype = None
+        L.zo_kv_quantize_int8.argtypes = [C.c_uint32] * 4 + [C.POINTER(C.c_int32), C.c_uint32, C.c_uint32, u16p, u16p, u32p, u16p]
         _lib = L
     return _lib
 
@@ -244,6 +246,16 @@ def slot_translate(ids, slot_map):
     out = np.empty_like(ids)
     lib().zo_slot_translate(_p(ids, C.c_uint32), _p(m, C.c_uint32), ids.size, _p(out, C.c_uint32))
     return out
+
+
+def kv_quantize_int8(kv_heads, head_dim, page_size, positions, pages_word_offset, scales_elem_offset, k_slot, v_slot, pages, scales):
+    """(pages u32, scales f16 bits) with every token's int8 rows and scales written in"""
+    pos = _c(positions, np.int32).ravel()
+    k, v = _c(k_slot, np.uint16).ravel(), _c(v_slot, np.uint16).ravel()
+    pg, sc = np.array(pages, np.uint32, copy=True).ravel(), np.array(scales, np.uint16, copy=True).ravel()
+    lib().zo_kv_quantize_int8(kv_heads, head_dim, page_size, pos.size, _p(pos, C.c_int32), pages_word_offset, scales_elem_offset,
+                              _p(k, C.c_uint16), _p(v, C.c_uint16), _p(pg, C.c_uint32), _p(sc, C.c_uint16))
+    return pg, sc
 
 
 def qkv_fused(affine, K, heads, kv_heads, head_dim, page_size, kv_page_stride, head_page_stride, v_page_offset,

@@ -32,6 +32,10 @@
  *                           multiplication by exp(i*freq), the cache as a reshaped
  *                           [page][K|V][kv_head][slot][dim] array; swapping the pair or the
  *                           sign of the sine, or writing V rotated, fails it
+ *   zo_kv_quantize_int8     numpy float32 formulation (np.rint, true division); the bound
+ *                           |q*scale - x| <= scale/2 + |x|*2^-11 on every element; an all-zero
+ *                           row; the reference test's own float64 reference within its +-1 count
+ *                           (tests/kernels/compile-qwen.mjs:720-747)
  * The reference's byte-exact repack fixtures (.weights-local/kernel-refs) are
  * git-ignored and absent, so fidelity of the plans to a real MLX checkpoint is
  * "parity unpinned"; what is pinned is each conversion against numpy.
@@ -313,6 +317,48 @@ ZO_API void zo_qkv_fused(uint32_t affine, uint32_t K, uint32_t heads, uint32_t k
                                          (size_t)slot * head_dim + pages_elem_offset + d + (group == 2 ? v_page_offset : 0);
         dst[0] = zo_f32_to_f16((float)lo);
         dst[half] = zo_f32_to_f16((float)hi);
+      }
+  }
+}
+
+/* ----------------------------------------------------- kv_quantize_int8 -- */
+
+/* int8 quantisation of one token's K and V rows into the paged int8 cache
+ * (src/compiler/shaders/kv_quantize_int8.wgsl:47-164), in the shader's f32 operations:
+ * per (kv head, side) scale = max|x| / 127, at least 1e-8, stored as f16;
+ * q = clamp(round-half-even(x * (1 / scale)), -127, 127), four to a word, low byte first.
+ * k_slot / v_slot are [tokens][kv_heads*head_dim] f16 bit patterns; pages and scales already
+ * hold the cache's previous contents. Layout: words page.head.slot.side.dim/4, scales
+ * page.head.slot.side (src/compiler/model-spec.ts:652-658). */
+ZO_API void zo_kv_quantize_int8(uint32_t kv_heads, uint32_t head_dim, uint32_t page_size, uint32_t tokens, const int32_t* positions,
+                                uint32_t pages_word_offset, uint32_t scales_elem_offset, const uint16_t* k_slot, const uint16_t* v_slot,
+                                uint32_t* pages, uint16_t* scales) {
+  const uint32_t row_words = head_dim / 4, kv_dim = kv_heads * head_dim;
+  for (uint32_t t = 0; t < tokens; t++) {
+    if (positions[t] < 0) continue;
+    const uint32_t page_no = (uint32_t)positions[t] / page_size, slot = (uint32_t)positions[t] % page_size;
+    for (uint32_t h = 0; h < kv_heads; h++)
+      for (uint32_t side = 0; side < 2; side++) {
+        const uint16_t* src = (side ? v_slot : k_slot) + (size_t)t * kv_dim + (size_t)h * head_dim;
+        float m = 0.f;
+        for (uint32_t d = 0; d < head_dim; d++) m = fmaxf(m, fabsf(zo_f16_to_f32(src[d])));
+        volatile float scale = m / 127.0f;
+        if (scale < 1e-8f) scale = 1e-8f;
+        volatile float inv = 1.0f / scale;
+        scales[(size_t)page_no * kv_heads * page_size * 2 + (size_t)h * page_size * 2 + slot * 2 + side + scales_elem_offset] =
+            zo_f32_to_f16(scale);
+        const size_t base = (size_t)page_no * kv_heads * page_size * 2 * row_words + (size_t)h * page_size * 2 * row_words +
+                            (size_t)slot * 2 * row_words + (size_t)side * row_words + pages_word_offset;
+        for (uint32_t w = 0; w < row_words; w++) {
+          uint32_t packed = 0;
+          for (int i = 0; i < 4; i++) {
+            volatile float prod = zo_f16_to_f32(src[4 * w + i]) * inv;
+            float q = nearbyintf(prod);  /* default rounding mode: ties to even */
+            q = q < -127.f ? -127.f : (q > 127.f ? 127.f : q);
+            packed |= ((uint32_t)(int32_t)q & 0xffu) << (8 * i);
+          }
+          pages[base + w] = packed;
+        }
       }
   }
 }

@@ -62,5 +62,28 @@ const put = (name) => { const b = load(name); const buf = dev.createBuffer(b.len
   try { dev.moeRouterTopk(idx, sc, logits, E, E + 1, true, true, 1) } catch (e) { threw = /K must be/.test(e.message) }
   if (!threw) throw new Error('top-k with K > E did not throw')
 }
+{
+  // fused QKV: the paged form, then the int8-KV pair (scratch rows + quantizer)
+  const { heads, kvHeads, headDim, d, pageSize, pages } = meta.qkv
+  const hps = pageSize * headDim, vpo = kvHeads * hps, kps = 2 * kvHeads * hps
+  const model = { d, affine: false, heads, kvHeads, headDim, pageSize, kvPageStride: kps, headPageStride: hps, vPageOffset: vpo, ropeTheta: 10000.0 }
+  const hidden = put('qx.bin'), scales = put('qs.bin'), weights = put('qw.bin'), pos = put('qpos.bin')
+  const q1 = dev.createBuffer(heads * headDim * 2, 'q'), kv = dev.createBuffer(pages * kps * 2, 'kv')
+  dev.fill(kv, 0)
+  dev.qkvFused([q1, kv, hidden, scales, weights, pos], dev.uniformBuf([0, 0]), model)
+  fs.writeFileSync(path.join(dir, 'q_paged.bin'), Buffer.from(dev.readBuffer(q1)))
+  fs.writeFileSync(path.join(dir, 'kv_paged.bin'), Buffer.from(dev.readBuffer(kv)))
+  const q2 = dev.createBuffer(heads * headDim * 2, 'q2'), ks = dev.createBuffer(kvHeads * headDim * 2, 'k_slot'), vs = dev.createBuffer(kvHeads * headDim * 2, 'v_slot')
+  dev.qkvFusedScratch([q2, ks, vs, hidden, scales, weights, pos], dev.uniformBuf([0, (heads + 2 * kvHeads) * headDim / 2]), model)
+  fs.writeFileSync(path.join(dir, 'q_scratch.bin'), Buffer.from(dev.readBuffer(q2)))
+  fs.writeFileSync(path.join(dir, 'k_slot.bin'), Buffer.from(dev.readBuffer(ks)))
+  fs.writeFileSync(path.join(dir, 'v_slot.bin'), Buffer.from(dev.readBuffer(vs)))
+  const rowWords = headDim / 4
+  const i8 = dev.createBuffer(pages * kvHeads * pageSize * 2 * rowWords * 4, 'kv_i8'), sc = dev.createBuffer(pages * kvHeads * pageSize * 2 * 2, 'kv_scales')
+  dev.fill(i8, 0); dev.fill(sc, 0)
+  dev.kvQuantizeInt8([ks, vs, i8, sc, pos], dev.uniformBuf([0, 0, 0, kvHeads * 2]), model)
+  fs.writeFileSync(path.join(dir, 'kv_i8.bin'), Buffer.from(dev.readBuffer(i8)))
+  fs.writeFileSync(path.join(dir, 'kv_sc.bin'), Buffer.from(dev.readBuffer(sc)))
+}
 dev.close()
 console.log('js gpu dispatch ok')

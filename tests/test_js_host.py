@@ -59,7 +59,16 @@ def test_js_dispatch_on_gpu(tmp_path, synth, oracle):
     for name, arr in (("rx", rx), ("rw", rw), ("rs", rs), ("rb", rb), ("gu", gu), ("slots", cslots), ("cscore", cscore),
                       ("gx", gx), ("gw", gw), ("gs", gs), ("gb", gb)):
         arr.tofile(str(tmp_path / (name + ".bin")))
+    # the fused QKV forms: paged, and scratch rows + int8 quantisation
+    QH, QKV, QHD, QK, QPAGE, QPOS = 4, 2, 64, 512, 8, 13
+    qrows = (QH + 2 * QKV) * QHD
+    qx, qw = synth.activations(1, QK, salt=9), synth.packed_weights(qrows, QK, salt=9)
+    qs = synth.scales(qrows, QK, affine=False, lo=0.01, hi=0.06, salt=9)
+    for name, arr in (("qx", qx), ("qw", qw), ("qs", qs), ("qpos", np.array([QPOS], np.int32))):
+        arr.tofile(str(tmp_path / (name + ".bin")))
     (tmp_path / "meta.json").write_text(json.dumps({"dense": {"K": K, "N": N},
+                                                    "qkv": {"heads": QH, "kvHeads": QKV, "headDim": QHD, "d": QK, "pageSize": QPAGE,
+                                                            "pages": 2},
                                                     "moe": {"E": E, "slots": slots, "tokens": tokens, "d": d, "ffn": ffn},
                                                     "block": {"D": D, "E": RE, "K": RK, "rowsS": rowsS, "F": F, "N2": N2, "S": S,
                                                               "GK": GK, "GF": GF}}))
@@ -88,3 +97,23 @@ def test_js_dispatch_on_gpu(tmp_path, synth, oracle):
     xv = gx.view(np.float16).astype(np.float64)[0]
     g, u = Wd[:GF] @ xv, Wd[GF:] @ xv
     assert rel_err(np.fromfile(str(tmp_path / "gated.bin"), np.float16).astype(np.float64), u * g / (1 + np.exp(-g)), 1e-2) < 1e-2
+    # fused QKV through the JS host: the paged form against the oracle, the scratch rows equal to the paged write,
+    # the int8 cache equal to the oracle's quantisation of those rows
+    hps, vpo, kps = QPAGE * QHD, QKV * QPAGE * QHD, 2 * QKV * QPAGE * QHD
+    want_q, want_p = oracle.qkv_fused(False, QK, QH, QKV, QHD, QPAGE, kps, hps, vpo, 0, 10000.0, QPOS, qx, qw, qs, None,
+                                      np.zeros(2 * kps, np.uint16))
+    got_q = np.fromfile(str(tmp_path / "q_paged.bin"), np.uint16)
+    got_p = np.fromfile(str(tmp_path / "kv_paged.bin"), np.uint16)
+    f = lambda a: a.view(np.float16).astype(np.float64)
+    assert np.max(np.abs(f(got_q) - f(want_q)) / (np.abs(f(want_q)) + 1e-3)) < 2e-2
+    assert np.max(np.abs(f(got_p) - f(want_p)) / (np.abs(f(want_p)) + 1e-3)) < 2e-2
+    paged = got_p.reshape(2, 2, QKV, QPAGE, QHD)
+    ks, vs = np.fromfile(str(tmp_path / "k_slot.bin"), np.uint16), np.fromfile(str(tmp_path / "v_slot.bin"), np.uint16)
+    assert np.array_equal(ks.reshape(QKV, QHD), paged[QPOS // QPAGE, 0, :, QPOS % QPAGE, :])
+    assert np.array_equal(vs.reshape(QKV, QHD), paged[QPOS // QPAGE, 1, :, QPOS % QPAGE, :])
+    assert np.array_equal(np.fromfile(str(tmp_path / "q_scratch.bin"), np.uint16), got_q)
+    rw4 = QHD // 4
+    want_pg, want_sc = oracle.kv_quantize_int8(QKV, QHD, QPAGE, [QPOS], 0, 0, ks, vs, np.zeros(2 * QKV * QPAGE * 2 * rw4, np.uint32),
+                                               np.zeros(2 * QKV * QPAGE * 2, np.uint16))
+    assert np.array_equal(np.fromfile(str(tmp_path / "kv_i8.bin"), np.uint32), want_pg)
+    assert np.array_equal(np.fromfile(str(tmp_path / "kv_sc.bin"), np.uint16), want_sc)

@@ -264,3 +264,82 @@ def test_qkv_fused(oracle, synth, affine):
     untouched[pos // page, :, :, pos % page] = False
     assert np.all(cache[untouched] == 0x1234), "only the position's slot is written"
     assert not close(q16.reshape(heads, hd), np.concatenate([rope(q)[:, half:], rope(q)[:, :half]], 1))
+
+
+# ---------------------------------------------------------------- kv_quantize_int8 ----------------------------
+
+def _kvq_case(kv_heads, head_dim, page_size, tokens, seed, scale=1.0):
+    rng = np.random.default_rng(seed)
+    k = (rng.uniform(-1, 1, (tokens, kv_heads * head_dim)) * scale).astype(np.float16)
+    v = (rng.uniform(-1, 1, (tokens, kv_heads * head_dim)) * scale).astype(np.float16)
+    return k, v
+
+
+def _kvq_numpy(kv_heads, head_dim, page_size, positions, k, v, pages, scales):
+    """Independent float32 formulation: vectorised numpy, np.rint, true division."""
+    rw = head_dim // 4
+    pages = pages.copy().reshape(-1, kv_heads, page_size, 2, rw)
+    scales = scales.copy().reshape(-1, kv_heads, page_size, 2)
+    for t, pos in enumerate(positions):
+        if pos < 0:
+            continue
+        page, slot = divmod(int(pos), page_size)
+        for side, src in enumerate((k, v)):
+            x = src[t].astype(np.float32).reshape(kv_heads, head_dim)
+            sc = np.maximum(np.abs(x).max(axis=1) / np.float32(127.0), np.float32(1e-8)).astype(np.float32)
+            inv = (np.float32(1.0) / sc).astype(np.float32)
+            q = np.clip(np.rint((x * inv[:, None]).astype(np.float32)), -127, 127).astype(np.int32)
+            b = (q & 0xFF).astype(np.uint32).reshape(kv_heads, rw, 4)
+            pages[page, :, slot, side, :] = b[..., 0] | (b[..., 1] << 8) | (b[..., 2] << 16) | (b[..., 3] << 24)
+            scales[page, :, slot, side] = sc.astype(np.float16).view(np.uint16)
+    return pages.ravel(), scales.ravel()
+
+
+@pytest.mark.parametrize("kv_heads,head_dim,page_size,tokens", [(8, 128, 16, 1), (2, 256, 16, 3), (3, 96, 8, 2), (1, 4, 4, 1)])
+def test_kv_quantize_int8_equals_numpy_and_bounds(oracle, kv_heads, head_dim, page_size, tokens):
+    k, v = _kvq_case(kv_heads, head_dim, page_size, tokens, 5 + head_dim)
+    k[0, :head_dim] = 0                                     # an all-zero row: scale clamps at 1e-8, which is 0 in f16
+    pages_n = 3
+    positions = np.array([2 * page_size + 1, 3, -1][:tokens], np.int32)   # page 2 slot 1, page 0 slot 3, a skipped token
+    rw = head_dim // 4
+    pages0 = np.full(pages_n * kv_heads * page_size * 2 * rw, 0xDEADBEEF, np.uint32)
+    scales0 = np.full(pages_n * kv_heads * page_size * 2, 0x7BFF, np.uint16)
+    pg, sc = oracle.kv_quantize_int8(kv_heads, head_dim, page_size, positions, 0, 0, k.view(np.uint16), v.view(np.uint16), pages0, scales0)
+    want_pg, want_sc = _kvq_numpy(kv_heads, head_dim, page_size, positions, k, v, pages0, scales0)
+    assert np.array_equal(pg, want_pg) and np.array_equal(sc, want_sc)
+    # the accuracy contract: |q*scale - x| <= scale/2 (+ the f16 rounding of the stored scale), and nothing else written
+    pgv = pg.reshape(pages_n, kv_heads, page_size, 2, rw)
+    scv = sc.view(np.float16).reshape(pages_n, kv_heads, page_size, 2).astype(np.float64)
+    touched = np.zeros(pgv.shape[:4], bool)
+    for t, pos in enumerate(positions):
+        if pos < 0:
+            continue
+        page, slot = divmod(int(pos), page_size)
+        for side, src in enumerate((k, v)):
+            words = pgv[page, :, slot, side, :]
+            q = np.stack([(words >> (8 * i)) & 0xFF for i in range(4)], axis=-1).astype(np.int64).reshape(kv_heads, head_dim)
+            q = np.where(q > 127, q - 256, q)
+            x = src[t].astype(np.float64).reshape(kv_heads, head_dim)
+            s = scv[page, :, slot, side][:, None]
+            assert np.all(np.abs(q * s - x) <= s / 2 + np.abs(x) * 2.0 ** -10 + 1e-12)
+            assert np.all(np.abs(q) <= 127)
+            # the reference test's own float64 reference, to its +-1 count (compile-qwen.mjs:720-747)
+            s64 = np.maximum(np.abs(x).max(axis=1, keepdims=True) / 127, 1e-8)
+            ref = np.clip(np.floor(x / s64 + 0.5), -127, 127)
+            assert np.max(np.abs(q - ref)) <= 1
+            touched[page, :, slot, side] = True
+    assert np.all(pgv[~touched] == 0xDEADBEEF) and np.all(sc.reshape(touched.shape)[~touched] == 0x7BFF)
+    assert sc.reshape(touched.shape)[int(positions[0]) // page_size, 0, int(positions[0]) % page_size, 0] == 0   # the zero row's scale
+
+
+def test_kv_quantize_int8_offsets(oracle):
+    kv_heads, head_dim, page_size = 2, 64, 4
+    k, v = _kvq_case(kv_heads, head_dim, page_size, 1, 9)
+    rw = head_dim // 4
+    n_words, n_sc = 2 * kv_heads * page_size * 2 * rw, 2 * kv_heads * page_size * 2
+    base_pg, base_sc = oracle.kv_quantize_int8(kv_heads, head_dim, page_size, [5], 0, 0, k.view(np.uint16), v.view(np.uint16),
+                                               np.zeros(n_words, np.uint32), np.zeros(n_sc, np.uint16))
+    off_pg, off_sc = oracle.kv_quantize_int8(kv_heads, head_dim, page_size, [5], 7, 3, k.view(np.uint16), v.view(np.uint16),
+                                             np.zeros(n_words + 7, np.uint32), np.zeros(n_sc + 3, np.uint16))
+    assert np.array_equal(off_pg[7:], base_pg) and not off_pg[:7].any()
+    assert np.array_equal(off_sc[3:], base_sc) and not off_sc[:3].any()

@@ -283,6 +283,70 @@ __global__ __launch_bounds__(64) void slot_translate_kernel(uint32_t* __restrict
   ids_out[i] = s == 0xffffffffu ? 0u : s;
 }
 
+// ---------------------------------------------------------------- kv_quantize_int8 ----
+// One wave per (token, kv head, side): max |x| over the head's row, scale = max / 127 (at least
+// 1e-8), q = clamp(round-half-even(x / scale)) packed four to a word, and the f16 scale
+// (src/compiler/shaders/kv_quantize_int8.wgsl:47-164). Page layout, in words:
+// page . head . slot . side(K|V) . dim/4; scales: page . head . slot . side.
+struct KvqParams {
+  uint32_t kv_heads, head_dim, page_size, tokens, pos_off, pages_word_off, scales_off;
+  uint64_t pages_capacity_words, scales_capacity;
+};
+constexpr int KVQ_TURNS = 4;  // words of a row per lane: head_dim <= 4 * 64 * KVQ_TURNS
+
+__global__ __launch_bounds__(256) void kv_quantize_int8_kernel(uint32_t* __restrict__ pages, _Float16* __restrict__ scales,
+                                                               const _Float16* __restrict__ k_slot, const _Float16* __restrict__ v_slot,
+                                                               const int32_t* __restrict__ position_map, const KvqParams p) {
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t unit = blockIdx.x * 4u + (threadIdx.x >> 6);  // uniform per wave
+  if (unit >= p.tokens * p.kv_heads * 2u) return;
+  const uint32_t tok = unit / (p.kv_heads * 2u), rest = unit - tok * p.kv_heads * 2u;
+  const uint32_t head = rest >> 1, side = rest & 1u;
+  const uint32_t row_words = p.head_dim / 4u;
+  const _Float16* src = (side ? v_slot : k_slot) + (size_t)tok * p.kv_heads * p.head_dim + (size_t)head * p.head_dim;
+  float v[KVQ_TURNS][4];
+  float m = 0.f;
+#pragma unroll
+  for (int t = 0; t < KVQ_TURNS; t++) {
+    const uint32_t w = lane + t * 64u;
+#pragma unroll
+    for (int i = 0; i < 4; i++) v[t][i] = 0.f;
+    if (w < row_words) {
+      const h4 x = *reinterpret_cast<const h4*>(src + 4u * w);
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        v[t][i] = (float)x[i];
+        m = fmaxf(m, fabsf(v[t][i]));
+      }
+    }
+  }
+  m = wave_max(m);
+  float scale = m / 127.0f;
+  if (scale < 1e-8f) scale = 1e-8f;
+  const float inv_scale = 1.0f / scale;
+  const int32_t position = position_map[p.pos_off + tok];
+  if (position < 0) return;  // uniform per wave
+  const uint32_t page_no = (uint32_t)position / p.page_size, slot = (uint32_t)position - page_no * p.page_size;
+  const uint64_t scale_idx = (uint64_t)page_no * p.kv_heads * p.page_size * 2u + (uint64_t)head * p.page_size * 2u + slot * 2u + side + p.scales_off;
+  if (lane == 0 && (!p.scales_capacity || scale_idx < p.scales_capacity)) scales[scale_idx] = (_Float16)scale;
+  const uint64_t base = (uint64_t)page_no * p.kv_heads * p.page_size * 2u * row_words + (uint64_t)head * p.page_size * 2u * row_words +
+                        (uint64_t)slot * 2u * row_words + (uint64_t)side * row_words + p.pages_word_off;
+#pragma unroll
+  for (int t = 0; t < KVQ_TURNS; t++) {
+    const uint32_t w = lane + t * 64u;
+    if (w < row_words && (!p.pages_capacity_words || base + w < p.pages_capacity_words)) {
+      uint32_t packed = 0;
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        float q = __builtin_rintf(v[t][i] * inv_scale);
+        q = fminf(fmaxf(q, -127.f), 127.f);
+        packed |= ((uint32_t)(int32_t)q & 0xffu) << (8 * i);
+      }
+      pages[base + w] = packed;
+    }
+  }
+}
+
 uint32_t grid_for(uint64_t threads) {
   uint64_t blocks = (threads + 255) / 256;
   return (uint32_t)(blocks > 16384 ? 16384 : (blocks ? blocks : 1));
@@ -340,6 +404,19 @@ hipError_t launch_router_topk(void* out_idx, void* out_score, const void* logits
   hipLaunchKernelGGL(router_topk_kernel, dim3((tokens + 3) / 4), dim3(256), 0, s, reinterpret_cast<uint32_t*>(out_idx),
                      reinterpret_cast<float*>(out_score), reinterpret_cast<const float*>(logits), E, K, norm_topk, has_shared,
                      tokens);
+  return hipGetLastError();
+}
+
+hipError_t launch_kv_quantize_int8(void* pages_i8, void* scales, const void* k_slot, const void* v_slot, const int32_t* position_map,
+                                   uint32_t kv_heads, uint32_t head_dim, uint32_t page_size, uint32_t tokens, uint32_t pos_off,
+                                   uint32_t pages_word_off, uint32_t scales_off, uint64_t pages_capacity_words, uint64_t scales_capacity,
+                                   hipStream_t s) {
+  if (head_dim > 4u * 64u * KVQ_TURNS) return hipErrorInvalidValue;  // rejected by the entry point
+  const KvqParams p{kv_heads, head_dim, page_size, tokens, pos_off, pages_word_off, scales_off, pages_capacity_words, scales_capacity};
+  const uint32_t units = tokens * kv_heads * 2u;
+  hipLaunchKernelGGL(kv_quantize_int8_kernel, dim3((units + 3) / 4), dim3(256), 0, s, reinterpret_cast<uint32_t*>(pages_i8),
+                     reinterpret_cast<_Float16*>(scales), reinterpret_cast<const _Float16*>(k_slot), reinterpret_cast<const _Float16*>(v_slot),
+                     position_map, p);
   return hipGetLastError();
 }
 

@@ -38,6 +38,8 @@ struct GemvParams {
   // QKV form: rows are RoPE pairs; the epilogue rotates and scatters into q_out / the paged KV cache
   _Float16* q_out;
   _Float16* kv_pages;
+  _Float16* k_slot;  // both set: K and V rows go here, [kv_heads*head_dim] each, instead of into kv_pages
+  _Float16* v_slot;
   const int32_t* position_map;
   uint32_t half_dim, head_dim, q_pairs, kv_pairs, q_dim, kv_dim;
   uint32_t page_size, kv_page_stride, head_page_stride, v_page_offset, pos_off, pages_off;
@@ -287,8 +289,10 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(const GemvParams p) {
               hi = c * second + sn * total;
             }
             const size_t at = cache + (q.group == 2 ? p.v_page_offset : 0u);
-            _Float16* dst = q.group == 0 ? p.q_out + (size_t)q.head * p.head_dim + q.dim_lo : p.kv_pages + at;
-            if (q.group == 0 || position >= 0 && (!p.kv_capacity || at + p.half_dim < p.kv_capacity)) {
+            const size_t in_row = (size_t)q.head * p.head_dim + q.dim_lo;
+            _Float16* dst = q.group == 0 ? p.q_out + in_row : p.kv_pages + at;
+            if (p.k_slot && q.group != 0) dst = (q.group == 1 ? p.k_slot : p.v_slot) + in_row;
+            if (q.group == 0 || p.k_slot || position >= 0 && (!p.kv_capacity || at + p.half_dim < p.kv_capacity)) {
               dst[0] = (_Float16)lo;
               dst[p.half_dim] = (_Float16)hi;
             }
@@ -361,11 +365,12 @@ hipError_t launch_gemv(const MatmulArgs& a, const Tune& t, hipStream_t s) {
   p.weights2 = a.up_weights; p.scales2 = a.up_scales; p.biases2 = a.up_biases;
   if (a.qkv) {
     const QkvArgs& q = *a.qkv;
-    p.q_out = q.q_out; p.kv_pages = q.kv_pages; p.position_map = q.position_map;
+    p.q_out = q.q_out; p.kv_pages = q.kv_pages; p.k_slot = q.k_slot; p.v_slot = q.v_slot; p.position_map = q.position_map;
     p.half_dim = q.head_dim / 2; p.head_dim = q.head_dim;
     p.q_pairs = q.heads * p.half_dim; p.kv_pairs = q.kv_heads * p.half_dim;
     p.q_dim = q.heads * q.head_dim; p.kv_dim = q.kv_heads * q.head_dim;
-    p.page_size = q.page_size; p.kv_page_stride = q.kv_page_stride; p.head_page_stride = q.head_page_stride;
+    // the scratch form has no pages; its cache address is computed and unused
+    p.page_size = q.page_size ? q.page_size : 1; p.kv_page_stride = q.kv_page_stride; p.head_page_stride = q.head_page_stride;
     p.v_page_offset = q.v_page_offset; p.pos_off = q.position_map_elem_offset; p.pages_off = q.pages_elem_offset;
     p.rope_theta = q.rope_theta; p.kv_capacity = q.kv_capacity;
   }

@@ -9,6 +9,8 @@ namespace ztvm {
 struct QkvArgs {
   _Float16* q_out;
   _Float16* kv_pages;
+  _Float16* k_slot = nullptr;  // both set: K and V go to two [kv_heads*head_dim] rows instead of the paged cache
+  _Float16* v_slot = nullptr;
   const int32_t* position_map;
   uint32_t heads, kv_heads, head_dim;
   uint32_t page_size, kv_page_stride, head_page_stride, v_page_offset;  // f16 elements
@@ -72,6 +74,10 @@ hipError_t launch_router_logits(void* logits, const void* x, const void* w, cons
 hipError_t launch_router_topk(void* out_idx, void* out_score, const void* logits, uint32_t E, uint32_t K, uint32_t norm_topk,
                               uint32_t has_shared, uint32_t tokens, hipStream_t s);
 uint32_t router_topk_max_experts();
+hipError_t launch_kv_quantize_int8(void* pages_i8, void* scales, const void* k_slot, const void* v_slot, const int32_t* position_map,
+                                   uint32_t kv_heads, uint32_t head_dim, uint32_t page_size, uint32_t tokens, uint32_t pos_off,
+                                   uint32_t pages_word_off, uint32_t scales_off, uint64_t pages_capacity_words, uint64_t scales_capacity,
+                                   hipStream_t s);
 hipError_t launch_slot_translate(void* ids_out, const void* ids_in, const void* slot_map, uint32_t n, uint32_t map_len, hipStream_t s);
 
 // load-time repacking of checkpoint records (repack.hip); convert: 0 raw, 1 bf16->f16, 2 bf16->f32

@@ -387,7 +387,9 @@ int ztvm_ffn_gated(ztvm_ctx* ctx, const ztvm_matmul_desc* desc, uint64_t up_weig
   return ZTVM_OK;
 }
 
-int ztvm_qkv_fused(ztvm_ctx* ctx, const ztvm_qkv_fused_desc* d) {
+// k_slot / v_slot non-zero: the int8-KV-mode variant, K and V go to two [kv_heads*head_dim] scratch rows
+static int qkv_fused_common(ztvm_ctx* ctx, const ztvm_qkv_fused_desc* d, uint64_t k_slot, uint64_t v_slot) {
+  const bool scratch = k_slot || v_slot;
   if (!ctx) return fail(nullptr, ZTVM_E_INVALID, "null context");
   if (!d) return fail(ctx, ZTVM_E_INVALID, "ztvm_qkv_fused: null descriptor");
   if (d->bits != 4) return fail(ctx, ZTVM_E_UNSUPPORTED, "ztvm_qkv_fused: 4-bit rows only (got %u)", d->bits);
@@ -402,13 +404,15 @@ int ztvm_qkv_fused(ztvm_ctx* ctx, const ztvm_qkv_fused_desc* d) {
     return fail(ctx, ZTVM_E_INVALID, "ztvm_qkv_fused: SCALES_PER_ROW=%u does not match K=%llu at group %u", d->scales_per_row, (unsigned long long)K, G);
   if ((uint64_t)(d->heads + 2u * d->kv_heads) * d->head_dim * d->k_packed * 4u >= (1ull << 31))
     return fail(ctx, ZTVM_E_INVALID, "ztvm_qkv_fused: the fused weight matrix must stay under 2 GiB");
-  if (!d->page_size || !d->kv_page_stride || !d->head_page_stride)
+  if (scratch) {
+    if (!k_slot || !v_slot || ((k_slot | v_slot) & 1u)) return fail(ctx, ZTVM_E_INVALID, "ztvm_qkv_fused_scratch: k_slot and v_slot must both be given, 2-byte aligned");
+  } else if (!d->page_size || !d->kv_page_stride || !d->head_page_stride) {
     return fail(ctx, ZTVM_E_INVALID, "ztvm_qkv_fused: page_size, kv_page_stride and head_page_stride must be > 0");
-  if ((uint64_t)d->page_size * d->head_dim > d->head_page_stride || (uint64_t)d->kv_heads * d->head_page_stride > d->v_page_offset ||
+  } else if ((uint64_t)d->page_size * d->head_dim > d->head_page_stride || (uint64_t)d->kv_heads * d->head_page_stride > d->v_page_offset ||
       (uint64_t)d->v_page_offset + (uint64_t)d->kv_heads * d->head_page_stride > d->kv_page_stride)
     return fail(ctx, ZTVM_E_INVALID, "ztvm_qkv_fused: page layout overlaps (page_size*head_dim <= head_page_stride, kv_heads*head_page_stride <= v_page_offset, v_page_offset + kv_heads*head_page_stride <= kv_page_stride)");
   if (!(d->rope_theta > 0.f)) return fail(ctx, ZTVM_E_INVALID, "ztvm_qkv_fused: rope_theta must be > 0");
-  if (!d->q_out || !d->kv_pages || !d->hidden || !d->scales || !d->weights || !d->position_map)
+  if (!d->q_out || (!scratch && !d->kv_pages) || !d->hidden || !d->scales || !d->weights || !d->position_map)
     return fail(ctx, ZTVM_E_INVALID, "ztvm_qkv_fused: null buffer");
   if (d->affine && !d->biases) return fail(ctx, ZTVM_E_INVALID, "ztvm_qkv_fused: affine rows have no bias buffer");
   if ((d->hidden | d->weights | d->scales | (d->affine ? d->biases : 0)) & 15u) return fail(ctx, ZTVM_E_INVALID, "ztvm_qkv_fused: hidden, weights, scales and biases must be 16-byte aligned");
@@ -420,6 +424,8 @@ int ztvm_qkv_fused(ztvm_ctx* ctx, const ztvm_qkv_fused_desc* d) {
   QkvArgs q{};
   q.q_out = reinterpret_cast<_Float16*>(d->q_out);
   q.kv_pages = reinterpret_cast<_Float16*>(d->kv_pages);
+  q.k_slot = reinterpret_cast<_Float16*>(k_slot);
+  q.v_slot = reinterpret_cast<_Float16*>(v_slot);
   q.position_map = reinterpret_cast<const int32_t*>(d->position_map);
   q.heads = d->heads; q.kv_heads = d->kv_heads; q.head_dim = d->head_dim;
   q.page_size = d->page_size; q.kv_page_stride = d->kv_page_stride; q.head_page_stride = d->head_page_stride;
@@ -440,6 +446,31 @@ int ztvm_qkv_fused(ztvm_ctx* ctx, const ztvm_qkv_fused_desc* d) {
   a.up_biases = d->affine ? a.biases + (size_t)half * d->scales_per_row : nullptr;
   a.qkv = &q;
   HIP_TRY(ctx, launch_gemv(a, ctx->tune, ctx->stream));
+  return ZTVM_OK;
+}
+
+int ztvm_qkv_fused(ztvm_ctx* ctx, const ztvm_qkv_fused_desc* d) { return qkv_fused_common(ctx, d, 0, 0); }
+
+int ztvm_qkv_fused_scratch(ztvm_ctx* ctx, const ztvm_qkv_fused_desc* d, uint64_t k_slot, uint64_t v_slot) {
+  if (!k_slot || !v_slot) return fail(ctx, ZTVM_E_INVALID, "ztvm_qkv_fused_scratch: null k_slot / v_slot");
+  return qkv_fused_common(ctx, d, k_slot, v_slot);
+}
+
+int ztvm_kv_quantize_int8(ztvm_ctx* ctx, const ztvm_kv_quantize_desc* d) {
+  if (!ctx) return fail(nullptr, ZTVM_E_INVALID, "null context");
+  if (!d) return fail(ctx, ZTVM_E_INVALID, "ztvm_kv_quantize_int8: null descriptor");
+  if (!d->kv_heads || !d->head_dim || (d->head_dim & 3u) || !d->page_size)
+    return fail(ctx, ZTVM_E_INVALID, "ztvm_kv_quantize_int8: kv_heads, page_size and a head_dim that is a multiple of 4 are required");
+  if (d->head_dim > 1024u) return fail(ctx, ZTVM_E_UNSUPPORTED, "ztvm_kv_quantize_int8: head_dim %u > 1024", d->head_dim);
+  if (!d->k_slot || !d->v_slot || !d->pages_i8 || !d->scales || !d->position_map) return fail(ctx, ZTVM_E_INVALID, "ztvm_kv_quantize_int8: null buffer");
+  if (((d->k_slot | d->v_slot) & 7u) || (d->pages_i8 & 3u) || (d->scales & 1u) || (d->position_map & 3u))
+    return fail(ctx, ZTVM_E_INVALID, "ztvm_kv_quantize_int8: misaligned buffer (slots 8, pages 4, scales 2, positions 4 bytes)");
+  if (((uint64_t)d->kv_heads * d->head_dim) & 3u) return fail(ctx, ZTVM_E_INVALID, "ztvm_kv_quantize_int8: kv_heads*head_dim must be a multiple of 4");
+  if (!d->tokens) return ZTVM_OK;
+  HIP_TRY(ctx, launch_kv_quantize_int8(reinterpret_cast<void*>(d->pages_i8), reinterpret_cast<void*>(d->scales), reinterpret_cast<const void*>(d->k_slot),
+                                       reinterpret_cast<const void*>(d->v_slot), reinterpret_cast<const int32_t*>(d->position_map), d->kv_heads,
+                                       d->head_dim, d->page_size, d->tokens, d->position_map_elem_offset, d->pages_word_offset,
+                                       d->scales_elem_offset, d->pages_capacity_words, d->scales_capacity, ctx->stream));
   return ZTVM_OK;
 }
 

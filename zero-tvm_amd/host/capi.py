@@ -16,7 +16,8 @@ E_INVALID, E_HIP, E_UNSUPPORTED, E_NODEVICE = -1, -2, -3, -4
 EXPORTS = [
     "ztvm_abi_version", "ztvm_last_error", "ztvm_create", "ztvm_destroy", "ztvm_device_info",
     "ztvm_alloc", "ztvm_free", "ztvm_upload", "ztvm_download", "ztvm_fill", "ztvm_copy", "ztvm_sync",
-    "ztvm_matmul_validate", "ztvm_matmul_resolve", "ztvm_matmul", "ztvm_ffn_gated", "ztvm_qkv_fused", "ztvm_dequant",
+    "ztvm_matmul_validate", "ztvm_matmul_resolve", "ztvm_matmul", "ztvm_ffn_gated", "ztvm_qkv_fused", "ztvm_qkv_fused_scratch",
+    "ztvm_kv_quantize_int8", "ztvm_dequant",
     "ztvm_record_begin", "ztvm_record_end", "ztvm_submit", "ztvm_cmdbuf_destroy",
     "ztvm_event_create", "ztvm_event_destroy", "ztvm_event_record", "ztvm_event_elapsed_ms",
     "ztvm_set_option", "ztvm_get_option",
@@ -48,6 +49,14 @@ class QkvFusedDesc(C.Structure):
         "head_page_stride", "v_page_offset", "position_map_elem_offset", "pages_elem_offset")] + [
         ("rope_theta", C.c_float), ("kv_capacity", C.c_uint64)] + [
         (n, C.c_uint64) for n in ("q_out", "kv_pages", "hidden", "scales", "weights", "position_map", "biases")]
+
+
+class KvQuantizeDesc(C.Structure):
+    """Mirror of ztvm_kv_quantize_desc."""
+    _fields_ = [(n, C.c_uint32) for n in (
+        "kv_heads", "head_dim", "page_size", "tokens", "position_map_elem_offset", "pages_word_offset", "scales_elem_offset",
+        "reserved")] + [(n, C.c_uint64) for n in (
+            "pages_capacity_words", "scales_capacity", "k_slot", "v_slot", "pages_i8", "scales", "position_map")]
 
 
 _lib = None
@@ -91,6 +100,8 @@ def load():
     u32, u64 = C.c_uint32, C.c_uint64
     L.ztvm_ffn_gated.argtypes = [vp, C.POINTER(MatmulDesc), u64, u64, u64]
     L.ztvm_qkv_fused.argtypes = [vp, C.POINTER(QkvFusedDesc)]
+    L.ztvm_qkv_fused_scratch.argtypes = [vp, C.POINTER(QkvFusedDesc), C.c_uint64, C.c_uint64]
+    L.ztvm_kv_quantize_int8.argtypes = [vp, C.POINTER(KvQuantizeDesc)]
     L.ztvm_silu_mul.argtypes = [vp, u64, u64, u32, u32]
     L.ztvm_moe_combine.argtypes = [vp, u64, u64, u64, u32, u32, u32]
     L.ztvm_moe_router_logits.argtypes = [vp, u64, u64, u64, u64, u64, u32, u32, u32, u32]
@@ -187,6 +198,12 @@ class Context:
 
     def qkv_fused(self, desc):
         self._chk(self._L.ztvm_qkv_fused(self._h, C.byref(desc)))
+
+    def qkv_fused_scratch(self, desc, k_slot, v_slot):
+        self._chk(self._L.ztvm_qkv_fused_scratch(self._h, C.byref(desc), k_slot, v_slot))
+
+    def kv_quantize_int8(self, desc):
+        self._chk(self._L.ztvm_kv_quantize_int8(self._h, C.byref(desc)))
 
     def dequant(self, desc):
         self._chk(self._L.ztvm_dequant(self._h, C.byref(desc)))

@@ -462,11 +462,9 @@ napi_value RepackDequantSplit(napi_env env, napi_callback_info info) {  // (ctx,
   return rc ? throw_ztvm(env, (ztvm_ctx*)p, rc, "ztvm_repack_dequant_split") : undefined(env);
 }
 
-napi_value QkvFused(napi_env env, napi_callback_info info) {  // (ctx, desc): keys are the ztvm_qkv_fused_desc field names
-  napi_value a[2];
-  void* p;
-  if (!get_args(env, info, 2, a) || !get_ptr(env, a[0], &p)) return nullptr;
-  ztvm_qkv_fused_desc d;
+// a JS object whose keys are the ztvm_qkv_fused_desc field names -> the descriptor
+bool read_qkv_desc(napi_env env, napi_value obj, ztvm_qkv_fused_desc& d) {
+  napi_value a[2] = {nullptr, obj};
   memset(&d, 0, sizeof d);
   struct F32 { const char* name; uint32_t ztvm_qkv_fused_desc::*field; };
   static const F32 u32s[] = {
@@ -485,7 +483,7 @@ napi_value QkvFused(napi_env env, napi_callback_info info) {  // (ctx, desc): ke
     napi_get_named_property(env, a[1], f.name, &v);
     if (napi_get_value_uint32(env, v, &(d.*(f.field))) != napi_ok) {
       napi_throw_type_error(env, nullptr, (std::string("ztvm addon: descriptor field '") + f.name + "' must be a number").c_str());
-      return nullptr;
+      return false;
     }
   }
   struct F64 { const char* name; uint64_t ztvm_qkv_fused_desc::*field; };
@@ -499,7 +497,7 @@ napi_value QkvFused(napi_env env, napi_callback_info info) {  // (ctx, desc): ke
     napi_has_named_property(env, a[1], f.name, &has);
     if (!has) continue;
     napi_get_named_property(env, a[1], f.name, &v);
-    if (!get_u64(env, v, &(d.*(f.field)))) return nullptr;
+    if (!get_u64(env, v, &(d.*(f.field)))) return false;
   }
   napi_value v;
   bool has = false;
@@ -510,8 +508,43 @@ napi_value QkvFused(napi_env env, napi_callback_info info) {  // (ctx, desc): ke
     napi_get_value_double(env, v, &t);
     d.rope_theta = (float)t;
   }
+  return true;
+}
+
+napi_value QkvFused(napi_env env, napi_callback_info info) {  // (ctx, desc)
+  napi_value a[2];
+  void* p;
+  ztvm_qkv_fused_desc d;
+  if (!get_args(env, info, 2, a) || !get_ptr(env, a[0], &p) || !read_qkv_desc(env, a[1], d)) return nullptr;
   int rc = ztvm_qkv_fused((ztvm_ctx*)p, &d);
   return rc ? throw_ztvm(env, (ztvm_ctx*)p, rc, "ztvm_qkv_fused") : undefined(env);
+}
+
+napi_value QkvFusedScratch(napi_env env, napi_callback_info info) {  // (ctx, desc, kSlot, vSlot)
+  napi_value a[4];
+  void* p;
+  uint64_t ks, vs;
+  ztvm_qkv_fused_desc d;
+  if (!get_args(env, info, 4, a) || !get_ptr(env, a[0], &p) || !read_qkv_desc(env, a[1], d) || !get_u64(env, a[2], &ks) ||
+      !get_u64(env, a[3], &vs))
+    return nullptr;
+  int rc = ztvm_qkv_fused_scratch((ztvm_ctx*)p, &d, ks, vs);
+  return rc ? throw_ztvm(env, (ztvm_ctx*)p, rc, "ztvm_qkv_fused_scratch") : undefined(env);
+}
+
+// (ctx, pagesI8, scales, kSlot, vSlot, positionMap, pagesCapacityWords, scalesCapacity,
+//  kvHeads, headDim, pageSize, tokens, positionMapElemOffset, pagesWordOffset, scalesElemOffset)
+napi_value KvQuantizeInt8(napi_env env, napi_callback_info info) {
+  void* p; uint64_t a[7]; uint32_t v[7];
+  if (!get_addr_u32(env, info, &p, a, v)) return nullptr;
+  ztvm_kv_quantize_desc d;
+  memset(&d, 0, sizeof d);
+  d.pages_i8 = a[0]; d.scales = a[1]; d.k_slot = a[2]; d.v_slot = a[3]; d.position_map = a[4];
+  d.pages_capacity_words = a[5]; d.scales_capacity = a[6];
+  d.kv_heads = v[0]; d.head_dim = v[1]; d.page_size = v[2]; d.tokens = v[3];
+  d.position_map_elem_offset = v[4]; d.pages_word_offset = v[5]; d.scales_elem_offset = v[6];
+  int rc = ztvm_kv_quantize_int8((ztvm_ctx*)p, &d);
+  return rc ? throw_ztvm(env, (ztvm_ctx*)p, rc, "ztvm_kv_quantize_int8") : undefined(env);
 }
 
 napi_value Init(napi_env env, napi_value exports) {
@@ -523,7 +556,8 @@ napi_value Init(napi_env env, napi_value exports) {
       {"recordEnd", RecordEnd}, {"submit", Submit}, {"cmdbufDestroy", CmdbufDestroy}, {"setOption", SetOption},
       {"siluMul", SiluMul}, {"moeCombine", MoeCombine}, {"moeRouterLogits", MoeRouterLogits}, {"moeRouterTopk", MoeRouterTopk},
       {"moeSlotTranslate", MoeSlotTranslate}, {"ffnGated", FfnGated}, {"repackPart", RepackPart},
-      {"repackPermuteRows", RepackPermuteRows}, {"repackDequantSplit", RepackDequantSplit}, {"qkvFused", QkvFused}};
+      {"repackPermuteRows", RepackPermuteRows}, {"repackDequantSplit", RepackDequantSplit}, {"qkvFused", QkvFused},
+      {"qkvFusedScratch", QkvFusedScratch}, {"kvQuantizeInt8", KvQuantizeInt8}};
   for (const E& e : table) {
     napi_value fn;
     if (napi_create_function(env, e.name, NAPI_AUTO_LENGTH, e.fn, nullptr, &fn) != napi_ok) return nullptr;

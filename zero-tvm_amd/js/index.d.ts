@@ -41,6 +41,10 @@ export declare class Device {
     wgX?: number, wgY?: number, wgZ?: number): void
   qkvFused(bufs: BindEntry[], pod: Uniform, model: { d: number; affine?: boolean; heads: number; kvHeads: number; headDim: number
     pageSize: number; kvPageStride: number; headPageStride: number; vPageOffset: number; ropeTheta: number }): void
+  qkvFusedScratch(bufs: BindEntry[], pod: Uniform, model: { d: number; affine?: boolean; heads: number; kvHeads: number
+    headDim: number; ropeTheta: number }): void
+  kvQuantizeInt8(bufs: BindEntry[], pod: Uniform, model: { kvHeads: number; headDim: number; pageSize: number },
+    tokens?: number): void
   beginEncoder(): void
   finishEncoder(): unknown
   submit(cmdbuf: unknown): void

@@ -283,6 +283,30 @@ class Device {
       position_map: a(bufs[5]), biases: bufs[6] ? a(bufs[6]) : 0n,
     })
   }
+  /**
+   * qkv_fused_scratch.wgsl (int8-KV mode): bindings [q_out, k_slot, v_slot, hidden, scales, weights, position_map,
+   * (biases)], the PODArgs {position_map_elem_offset, packGridDimX} and the model constants of the shader prelude.
+   */
+  qkvFusedScratch(bufs, pod, model) {
+    const a = (b) => this._a(b)
+    const K = model.d
+    addon().qkvFusedScratch(this.ctx, {
+      bits: 4, affine: model.affine ? 1 : 0, k_packed: K / 8, scales_per_row: K / (model.affine ? 64 : 32),
+      heads: model.heads, kv_heads: model.kvHeads, head_dim: model.headDim, position_map_elem_offset: pod.words[0],
+      rope_theta: model.ropeTheta, q_out: a(bufs[0]), hidden: a(bufs[3]), scales: a(bufs[4]), weights: a(bufs[5]),
+      position_map: a(bufs[6]), biases: bufs[7] ? a(bufs[7]) : 0n,
+    }, a(bufs[1]), a(bufs[2]))
+  }
+  /**
+   * kv_quantize_int8.wgsl: bindings [k_slot, v_slot, pages_i8, scales, position_map], the PODArgs
+   * {position_map_elem_offset, pages_elem_offset (words), scales_elem_offset, packGridDimX}; tokens = grid y.
+   */
+  kvQuantizeInt8(bufs, pod, model, tokens) {
+    const w = pod.words, a = (b) => this._a(b)
+    addon().kvQuantizeInt8(this.ctx, a(bufs[2]), a(bufs[3]), a(bufs[0]), a(bufs[1]), a(bufs[4]),
+      BigInt(Math.floor(bufs[2].size / 4)), BigInt(Math.floor(bufs[3].size / 2)),
+      model.kvHeads, model.headDim, model.pageSize, tokens === undefined ? 1 : tokens, w[0], w[1], w[2])
+  }
   beginEncoder() { addon().recordBegin(this.ctx) }
   finishEncoder() { return addon().recordEnd(this.ctx) }
   submit(cmdbuf) { addon().submit(this.ctx, cmdbuf) }
