@@ -322,6 +322,15 @@ def main():
                   + synth.weight_bytes(4096, 14336))
         extra["decode_layer_8b_four_dispatches"] = {"us": round(ms * 1e3, 2), "GB/s": round(lbytes / ms / 1e6, 1),
                                                     "hbm_frac": round(lbytes / ms / 1e6 / HBM_PEAK_GBS, 4), "weight_MB": round(lbytes / 1e6, 1)}
+        # gate + up + SiLU at the 8B layer shape, plain and with the add + RMSNorm prologue folded in
+        dl, gm = _put(ctx, (synth.activations(1, 4096, salt=77).view(np.float16) * 0.3).astype(np.float16)), \
+            _put(ctx, np.full(4096, 1.0, np.float16))
+        ms_g = timed_graph(ctx, [lambda L=lsets[j % 6]: ctx.ffn_gated(L[2], *L[3]) for j in range(60)]) / 60
+        ms_p = timed_graph(ctx, [lambda L=lsets[j % 6]: ctx.ffn_gated_prologue(L[2], *L[3], dl, gm, 1e-5) for j in range(60)]) / 60
+        gbytes = 2 * synth.weight_bytes(14336, 4096)
+        extra["ffn_gated_K4096_N14336"] = {"us": round(ms_g * 1e3, 2), "GB/s": round(gbytes / ms_g / 1e6, 1),
+                                           "hbm_frac": round(gbytes / ms_g / 1e6 / HBM_PEAK_GBS, 4),
+                                           "with_add_rmsnorm_prologue_us": round(ms_p * 1e3, 2)}
         # small batches: the row-group GEMV (M <= 16) and the weight-streaming matrix-core kernel (M <= 128); int4,
         # configs[4]'s int3 M=8, and 8-bit rows
         for bits, M in ((4, 2), (4, 4), (4, 8), (4, 16), (4, 32), (4, 128), (3, 8), (8, 8), (8, 128)):

@@ -168,6 +168,16 @@ ZTVM_API int ztvm_matmul(ztvm_ctx* ctx, const ztvm_matmul_desc* desc);
 ZTVM_API int ztvm_ffn_gated(ztvm_ctx* ctx, const ztvm_matmul_desc* desc, uint64_t up_weights, uint64_t up_scales,
                             uint64_t up_biases);
 
+/* fused_ffn_prologue / fused_ffn_tiled_sg_prologue (src/compiler/shaders/fused_ffn_prologue.wgsl:1-165):
+ * ztvm_ffn_gated with the FFN-entry add + RMSNorm folded in. desc->in is the running residual
+ * [K] f16, delta the o-proj output to be added, gamma the norm gain:
+ *   val = f16(residual + delta);  x = f16(f32(val) * (1 / sqrt(mean(val^2) + rms_eps)) * f32(gamma))
+ * with the sum of squares in f32, and x feeds the gate / up dot products exactly as the stored
+ * normed vector did. One dense row (M = 1, the decode step), 4-bit symmetric (the reference's),
+ * 4-bit affine or 3-bit. Like the reference's kernel it does not write the residual sum anywhere. */
+ZTVM_API int ztvm_ffn_gated_prologue(ztvm_ctx* ctx, const ztvm_matmul_desc* desc, uint64_t up_weights, uint64_t up_scales,
+                                     uint64_t up_biases, uint64_t delta, uint64_t gamma, float rms_eps);
+
 /* QKV matmul + RoPE + KV append in one dispatch, decode path (one token). Replaces
  * qkv_fused / _sg / _sg_vec4 / _tiled_sg / _tiled2sg (src/compiler/shaders/qkv_fused.wgsl:23-193;
  * dispatch site src/zero-tvm/engine-core.ts:2320): bindings 0 q_out, 1 kv_pages, 2 hidden,

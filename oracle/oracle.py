@@ -67,6 +67,7 @@ def lib():
         L.zo_slot_translate.restype, L.zo_slot_translate.argtypes = None, [u32p, u32p, C.c_uint32, u32p]
         L.zo_qkv_fused.restype = None
         L.zo_qkv_fused.argtypes = [C.c_uint32] * 10 + [C.c_double, C.c_int32, u16p, u32p, u16p, u16p, u16p, u16p]
+        L.zo_add_rmsnorm.restype, L.zo_add_rmsnorm.argtypes = None, [u16p, u16p, u16p, C.c_uint32, C.c_float, u16p]
         L.zo_kv_quantize_int8.restype = None
         L.zo_kv_quantize_int8.argtypes = [C.c_uint32] * 4 + [C.POINTER(C.c_int32), C.c_uint32, C.c_uint32, u16p, u16p, u32p, u16p]
         _lib = L
@@ -245,6 +246,14 @@ def slot_translate(ids, slot_map):
     ids, m = _c(ids, np.uint32).ravel(), _c(slot_map, np.uint32).ravel()
     out = np.empty_like(ids)
     lib().zo_slot_translate(_p(ids, C.c_uint32), _p(m, C.c_uint32), ids.size, _p(out, C.c_uint32))
+    return out
+
+
+def add_rmsnorm(residual, delta, gamma, eps):
+    """f16 bits of RMSNorm(residual + delta) * gamma, the fused-FFN prologue's numerics"""
+    r, d, g = _c(residual, np.uint16).ravel(), _c(delta, np.uint16).ravel(), _c(gamma, np.uint16).ravel()
+    out = np.empty_like(r)
+    lib().zo_add_rmsnorm(_p(r, C.c_uint16), _p(d, C.c_uint16), _p(g, C.c_uint16), r.size, C.c_float(eps), _p(out, C.c_uint16))
     return out
 
 

@@ -36,6 +36,9 @@
  *                           |q*scale - x| <= scale/2 + |x|*2^-11 on every element; an all-zero
  *                           row; the reference test's own float64 reference within its +-1 count
  *                           (tests/kernels/compile-qwen.mjs:720-747)
+ *   zo_add_rmsnorm          numpy formulation (float64 sum of squares rounded once, float32 after:
+ *                           equal bit for bit); a constant row (closed form
+ *                           c / sqrt(c^2 + eps) * gamma); zero input; gamma = 1 gives unit RMS
  * The reference's byte-exact repack fixtures (.weights-local/kernel-refs) are
  * git-ignored and absent, so fidelity of the plans to a real MLX checkpoint is
  * "parity unpinned"; what is pinned is each conversion against numpy.
@@ -360,5 +363,33 @@ ZO_API void zo_kv_quantize_int8(uint32_t kv_heads, uint32_t head_dim, uint32_t p
           pages[base + w] = packed;
         }
       }
+  }
+}
+
+/* ------------------------------------------------------- add + RMSNorm -- */
+
+/* The FFN-entry add + RMSNorm as the fused-FFN prologue computes it
+ * (src/compiler/shaders/fused_ffn_prologue.wgsl:62-97, the numerics of add_norm.wgsl):
+ * val = f16(residual + delta); sum of f32(val)^2 in f32; rms_inv = 1 / sqrt(sum / K + eps);
+ * out = f16(f32(val) * rms_inv * f32(gamma)). The order of the f32 sum is the implementation's (a
+ * 64-lane tree in the shader, a wave-then-workgroup tree in the HIP kernel); every such order lies
+ * within a few f32 steps of the exactly rounded sum, which is what this function uses (the squares
+ * are exact in f32, so the double sum rounded once is that value). rms_inv may therefore differ from
+ * a kernel's in its last bits, and out by one f16 step on the rare element at a rounding boundary. */
+ZO_API void zo_add_rmsnorm(const uint16_t* residual, const uint16_t* delta, const uint16_t* gamma, uint32_t K, float eps,
+                           uint16_t* out) {
+  double exact = 0.0;
+  for (uint32_t k = 0; k < K; k++) {
+    const float val = zo_f16_to_f32(zo_f32_to_f16(zo_f16_to_f32(residual[k]) + zo_f16_to_f32(delta[k])));
+    exact += (double)val * (double)val;
+  }
+  volatile float ss = (float)exact;
+  volatile float mean = ss / (float)K;
+  const float rms_inv = 1.0f / sqrtf(mean + eps);
+  for (uint32_t k = 0; k < K; k++) {
+    const float val = zo_f16_to_f32(zo_f32_to_f16(zo_f16_to_f32(residual[k]) + zo_f16_to_f32(delta[k])));
+    volatile float t = val * rms_inv;
+    volatile float u = t * zo_f16_to_f32(gamma[k]);
+    out[k] = zo_f32_to_f16(u);
   }
 }

@@ -58,6 +58,12 @@ const put = (name) => { const b = load(name); const buf = dev.createBuffer(b.len
   dev.ffnGated(pipe, group, { buffer: gw, offset: GF * kp * 4, size: GF * kp * 4 }, { buffer: gs, offset: GF * spr * 2, size: GF * spr * 2 },
     { buffer: gb, offset: GF * spr * 2, size: GF * spr * 2 }, GF / 4)
   fs.writeFileSync(path.join(dir, 'gated.bin'), Buffer.from(dev.readBuffer(go)))
+  // the same dispatch with the add + RMSNorm prologue: binding 1 is the residual
+  const go2 = dev.createBuffer(GF * 2, 'gated_prologue')
+  const group2 = dev.bg(pipe, [go2, put('pres.bin'), gs, gw, dev.uniformBuf(z.densePod(GK, GF)), gb])
+  dev.ffnGatedPrologue(pipe, group2, { buffer: gw, offset: GF * kp * 4, size: GF * kp * 4 }, { buffer: gs, offset: GF * spr * 2, size: GF * spr * 2 },
+    { buffer: gb, offset: GF * spr * 2, size: GF * spr * 2 }, put('pdelta.bin'), put('pgamma.bin'), 1e-5, GF / 4)
+  fs.writeFileSync(path.join(dir, 'gated_prologue.bin'), Buffer.from(dev.readBuffer(go2)))
   let threw = false
   try { dev.moeRouterTopk(idx, sc, logits, E, E + 1, true, true, 1) } catch (e) { threw = /K must be/.test(e.message) }
   if (!threw) throw new Error('top-k with K > E did not throw')

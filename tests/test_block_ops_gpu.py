@@ -273,6 +273,78 @@ def test_ffn_gated_dense(ctx, capi, synth, oracle, bits, affine, M, N, K):
     assert not got[M].any()
 
 
+def _prologue_run(ctx, capi, bits, affine, N, K, res, dlt, gam, eps, w, s, b, normed):
+    kp, spr = K * bits // 32, K // (64 if affine else 32)
+    with Dev(ctx) as d:
+        out, out2 = d.empty(2 * N * 2, fill=0), d.empty(N * 2, fill=0)
+        W, S, B = d.put(w), d.put(s), (d.put(b) if affine else 0)
+        common = dict(bits=bits, affine=int(affine), M=1, N=N, k_packed=kp, scales_per_row=spr, weights=W, scales=S, biases=B)
+        ups = (W + N * kp * 4, S + N * spr * 2, B + N * spr * 2 if affine else 0)
+        ctx.ffn_gated_prologue(capi.MatmulDesc(out=out, in_=d.put(res), **common), *ups, d.put(dlt), d.put(gam), eps)
+        ctx.ffn_gated(capi.MatmulDesc(out=out2, in_=d.put(normed), **common), *ups)
+        got = ctx.download(out, 2 * N * 2, np.uint16).reshape(2, N)
+        return got, ctx.download(out2, N * 2, np.uint16)
+
+
+def test_ffn_gated_prologue_reference_case(ctx, capi, oracle):
+    """The reference's own test of the kernel (tests/kernels/run.mjs:1021-1072): Phi-3 width, eight output rows,
+    residual and delta uniform in +-0.75, gamma in 0.75..1.25, scales in 0.01..0.06, float64 sum of squares in the
+    reference, bar |got-ref| / (|ref| + 1e-3) < 2e-2."""
+    rng = np.random.default_rng(8)
+    K, N, eps = 3072, 8, 1e-5
+    res = (rng.random(K) * 1.5 - 0.75).astype(np.float16)
+    dlt = (rng.random(K) * 1.5 - 0.75).astype(np.float16)
+    gam = (rng.random(K) * 0.5 + 0.75).astype(np.float16)
+    w = rng.integers(0, 2 ** 32, (2 * N, K // 8), dtype=np.uint64).astype(np.uint32)
+    s = (rng.random((2 * N, K // 32)) * 0.05 + 0.01).astype(np.float16).view(np.uint16)
+    summed = (res.astype(np.float32) + dlt.astype(np.float32)).astype(np.float16).astype(np.float64)
+    normed64 = (summed / np.sqrt(np.mean(summed * summed) + eps) * gam.astype(np.float64)).astype(np.float16)
+    got, _ = _prologue_run(ctx, capi, 4, False, N, K, res, dlt, gam, eps, w, s, None, normed64.view(np.uint16))
+    ref = gated_reference(oracle, 4, False, N, K, normed64.view(np.uint16).reshape(1, K), w[:N], s[:N], None, w[N:], s[N:], None)[0]
+    assert np.max(np.abs(f16(got[0]) - ref) / (np.abs(ref) + 1e-3)) < 2e-2
+
+
+@pytest.mark.parametrize("bits,affine", [(4, False), (4, True), (3, True)])
+@pytest.mark.parametrize("N,K", [(8192, 3072), (100, 512), (64, 64), (130, 14336)])
+def test_ffn_gated_prologue(ctx, capi, synth, oracle, bits, affine, N, K):
+    """The fused FFN with the add + RMSNorm prologue at the reference kernel's shape (D = 3072, FFN_DIM = 8192) and
+    others, against the float64 reference on the oracle's normed vector and against the plain gated form fed that
+    vector. The normed vector is f16 and the sum of squares is f32: its summation order (index order in the oracle, a
+    tree in the kernel, another tree in the shader) moves 1/sqrt by a few f32 steps, which flips the f16 rounding of a
+    handful of the K normed values by one step. An output near zero whose up factor is large sees that as an absolute
+    error, so the floor of the relative bar is tied to the output scale: |got-ref| / (|ref| + 0.05*rms(ref)) < 1e-2."""
+    rng = np.random.default_rng(N + K)
+    res = rng.standard_normal(K).astype(np.float16)
+    dlt = (rng.standard_normal(K) * 0.3).astype(np.float16)
+    gam = (1 + 0.1 * rng.standard_normal(K)).astype(np.float16)
+    eps = 1e-5
+    w = synth.packed_weights(2 * N, K, bits=bits)
+    s = synth.scales(2 * N, K, affine=affine)
+    b = synth.biases(2 * N, K, s, "A") if affine else None
+    normed = oracle.add_rmsnorm(res.view(np.uint16), dlt.view(np.uint16), gam.view(np.uint16), eps)
+    got, two_step = _prologue_run(ctx, capi, bits, affine, N, K, res, dlt, gam, eps, w, s, b, normed)
+    ref = gated_reference(oracle, bits, affine, N, K, normed.reshape(1, K), w[:N], s[:N], b[:N] if affine else None, w[N:], s[N:],
+                          b[N:] if affine else None)[0]
+    floor = 0.05 * np.sqrt(np.mean(ref * ref))
+    assert np.max(np.abs(f16(got[0]) - ref) / (np.abs(ref) + floor)) < 1e-2
+    assert not got[1].any()
+    assert np.max(np.abs(f16(got[0]) - f16(two_step)) / (np.abs(f16(two_step)) + floor)) < 2e-3
+    # and most outputs are the same f16 value as the two-dispatch form gives
+    assert np.mean(got[0] == two_step) > 0.9
+
+
+def test_ffn_gated_prologue_rejects(ctx, capi):
+    p = 0x10000
+    desc = capi.MatmulDesc(bits=4, affine=0, M=1, N=64, k_packed=64, scales_per_row=16, out=p, in_=p, weights=p, scales=p)
+    for kw, args, needle in ((dict(), (p, p, 0, 0, p, 1e-5), "delta and gamma"), (dict(), (p, p, 0, p, p + 2, 1e-5), "aligned"),
+                             (dict(M=2), (p, p, 0, p, p, 1e-5), "one dense activation row"),
+                             (dict(), (p, p, 0, p, p, -1.0), "rms_eps"),
+                             (dict(bits=8, affine=1, k_packed=128, scales_per_row=8, biases=p), (p, p, p, p, p, 1e-5), "8-bit")):
+        dsc = capi.MatmulDesc(**{**{f[0]: getattr(desc, f[0]) for f in desc._fields_}, **kw})
+        with pytest.raises(capi.ZtvmError, match=needle):
+            ctx.ffn_gated_prologue(dsc, *args)
+
+
 def test_ffn_gated_moe_matches_three_dispatches(ctx, capi, synth, oracle):
     """Per (token, slot) pair on expert stacks: the one-pass form against gate, up and silu_mul dispatched
     separately (which round gate and up to f16 in between) and against the float64 formula."""

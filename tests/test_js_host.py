@@ -56,8 +56,11 @@ def test_js_dispatch_on_gpu(tmp_path, synth, oracle):
     cscore = rng.random((1, S)).astype(np.float32)
     gx, gw, gs = synth.activations(1, GK, salt=7), synth.packed_weights(2 * GF, GK, salt=7), synth.scales(2 * GF, GK, salt=7)
     gb = synth.biases(2 * GF, GK, gs, salt=7)
+    pres = rng.standard_normal(GK).astype(np.float16)
+    pdelta = (rng.standard_normal(GK) * 0.3).astype(np.float16)
+    pgamma = (1 + 0.1 * rng.standard_normal(GK)).astype(np.float16)
     for name, arr in (("rx", rx), ("rw", rw), ("rs", rs), ("rb", rb), ("gu", gu), ("slots", cslots), ("cscore", cscore),
-                      ("gx", gx), ("gw", gw), ("gs", gs), ("gb", gb)):
+                      ("gx", gx), ("gw", gw), ("gs", gs), ("gb", gb), ("pres", pres), ("pdelta", pdelta), ("pgamma", pgamma)):
         arr.tofile(str(tmp_path / (name + ".bin")))
     # the fused QKV forms: paged, and scratch rows + int8 quantisation
     QH, QKV, QHD, QK, QPAGE, QPOS = 4, 2, 64, 512, 8, 13
@@ -97,6 +100,11 @@ def test_js_dispatch_on_gpu(tmp_path, synth, oracle):
     xv = gx.view(np.float16).astype(np.float64)[0]
     g, u = Wd[:GF] @ xv, Wd[GF:] @ xv
     assert rel_err(np.fromfile(str(tmp_path / "gated.bin"), np.float16).astype(np.float64), u * g / (1 + np.exp(-g)), 1e-2) < 1e-2
+    xn = oracle.add_rmsnorm(pres.view(np.uint16), pdelta.view(np.uint16), pgamma.view(np.uint16), 1e-5).view(np.float16).astype(np.float64)
+    gp, upj = Wd[:GF] @ xn, Wd[GF:] @ xn
+    refp = upj * gp / (1 + np.exp(-gp))
+    gotp = np.fromfile(str(tmp_path / "gated_prologue.bin"), np.float16).astype(np.float64)
+    assert np.max(np.abs(gotp - refp) / (np.abs(refp) + 0.05 * np.sqrt(np.mean(refp * refp)))) < 1e-2
     # fused QKV through the JS host: the paged form against the oracle, the scratch rows equal to the paged write,
     # the int8 cache equal to the oracle's quantisation of those rows
     hps, vpo, kps = QPAGE * QHD, QKV * QPAGE * QHD, 2 * QKV * QPAGE * QHD

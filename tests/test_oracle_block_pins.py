@@ -343,3 +343,39 @@ def test_kv_quantize_int8_offsets(oracle):
                                              np.zeros(n_words + 7, np.uint32), np.zeros(n_sc + 3, np.uint16))
     assert np.array_equal(off_pg[7:], base_pg) and not off_pg[:7].any()
     assert np.array_equal(off_sc[3:], base_sc) and not off_sc[:3].any()
+
+
+# ---------------------------------------------------------------- add + RMSNorm -------------------------------
+
+def test_add_rmsnorm_against_numpy_and_closed_forms(oracle):
+    rng = np.random.default_rng(31)
+    K, eps = 3072, 1e-5
+    res = rng.standard_normal(K).astype(np.float16)
+    dlt = (rng.standard_normal(K) * 0.3).astype(np.float16)
+    gam = (1 + 0.1 * rng.standard_normal(K)).astype(np.float16)
+    got = oracle.add_rmsnorm(res.view(np.uint16), dlt.view(np.uint16), gam.view(np.uint16), eps).view(np.float16)
+    val = (res.astype(np.float32) + dlt.astype(np.float32)).astype(np.float16).astype(np.float32)
+    ss = np.float32(np.sum(val.astype(np.float64) ** 2))           # the exactly rounded sum of the (exact) squares
+    inv = np.float32(1.0) / np.sqrt(np.float32(ss / np.float32(K)) + np.float32(eps))
+    want = ((val * inv).astype(np.float32) * gam.astype(np.float32)).astype(np.float16)
+    assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+    # any float32 summation order lands within a rounding step of it on all but a handful of elements
+    inv32 = np.float32(1.0) / np.sqrt(np.float32(np.sum(val * val, dtype=np.float32) / np.float32(K)) + np.float32(eps))
+    other = ((val * inv32).astype(np.float32) * gam.astype(np.float32)).astype(np.float16)
+    ulp = np.abs(got.view(np.int16).astype(np.int32) - other.view(np.int16).astype(np.int32))
+    assert ulp.max() <= 1 and (ulp > 0).mean() < 0.02
+    # float64 truth, to f16 accuracy
+    v64 = val.astype(np.float64)
+    t64 = v64 / np.sqrt(np.mean(v64 * v64) + eps) * gam.astype(np.float64)
+    assert np.max(np.abs(got.astype(np.float64) - t64) / (np.abs(t64) + 1e-3)) < 1e-3
+    # a constant row: c / sqrt(c^2 + eps) * gamma; zeros stay zero; gamma = 1 gives unit RMS
+    c = np.full(K, 0.75, np.float16)
+    z = np.zeros(K, np.float16)
+    one = np.ones(K, np.float16)
+    got = oracle.add_rmsnorm(c.view(np.uint16), z.view(np.uint16), gam.view(np.uint16), eps).view(np.float16).astype(np.float64)
+    assert np.max(np.abs(got - 0.75 / np.sqrt(0.75 ** 2 + eps) * gam.astype(np.float64))) < 1e-3
+    assert not oracle.add_rmsnorm(z.view(np.uint16), z.view(np.uint16), gam.view(np.uint16), eps).any()
+    unit = oracle.add_rmsnorm(res.view(np.uint16), dlt.view(np.uint16), one.view(np.uint16), 0.0).view(np.float16).astype(np.float64)
+    assert abs(np.sqrt(np.mean(unit * unit)) - 1.0) < 1e-3
+    # the sum is over residual + delta, not either alone
+    assert not np.array_equal(oracle.add_rmsnorm(res.view(np.uint16), z.view(np.uint16), gam.view(np.uint16), eps), got)

@@ -32,6 +32,10 @@ struct GemvParams {
   const uint32_t* weights;
   const _Float16* biases;
   const uint32_t* ids;
+  // prologue form: `in` is the residual; x = RMSNorm(residual + delta) * gamma is formed while x is staged
+  const _Float16* delta;
+  const _Float16* gamma;
+  float rms_eps;
   const _Float16* scales2;   // gated form: the up projection's scales / weights / biases (same shape as the gate's)
   const uint32_t* weights2;
   const _Float16* biases2;
@@ -88,7 +92,13 @@ __device__ __forceinline__ QkvPair qkv_pair(const GemvParams& p, uint32_t pair) 
   return r;
 }
 
-template <int BITS, bool AFFINE, int LPR, int ROWS, int MAXT, bool GATED = false, bool QKV = false>
+//
+// PROLOGUE (a GATED launch): the FFN-entry add + RMSNorm is folded into the staging of x
+// (src/compiler/shaders/fused_ffn_prologue.wgsl:62-97): val = f16(residual + delta), the sum of
+// val^2 in f32 over the whole row, x = f16(f32(val) * (1 / sqrt(mean + eps)) * f32(gamma)).
+// Every workgroup recomputes the norm of the whole row; the add_norm dispatch and the round trip
+// of the normed vector through memory disappear.
+template <int BITS, bool AFFINE, int LPR, int ROWS, int MAXT, bool GATED = false, bool QKV = false, bool PROLOGUE = false>
 __global__ __launch_bounds__(MAXT) void gemv_kernel(const GemvParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
   constexpr int SUB = 64 / LPR;          // row slots per wave load
@@ -190,20 +200,65 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(const GemvParams p) {
   h8* xs_pieces = reinterpret_cast<h8*>(smem);
   const uint32_t padded_chunks = (p.nchunks + 63u) & ~63u;
   float* xsum = reinterpret_cast<float*>(smem + (size_t)padded_chunks * 64u);
-  for (uint32_t c = tid; c < p.nchunks; c += blockDim.x) {
-    float s = 0.f;
-    const h8* src = reinterpret_cast<const h8*>(x + (size_t)c * 32u);
+  if constexpr (!PROLOGUE) {
+    for (uint32_t c = tid; c < p.nchunks; c += blockDim.x) {
+      float s = 0.f;
+      const h8* src = reinterpret_cast<const h8*>(x + (size_t)c * 32u);
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-      const h8 v = src[j];
-      h8 o;
+      for (int j = 0; j < 4; j++) {
+        const h8 v = src[j];
+        h8 o;
 #pragma unroll
-      for (int sl = 0; sl < 8; sl++) o[sl] = v[BITS == 8 ? value_in_slot8(sl) : value_in_slot(sl)];
-      xs_pieces[x_slot(c, j)] = o;
+        for (int sl = 0; sl < 8; sl++) o[sl] = v[BITS == 8 ? value_in_slot8(sl) : value_in_slot(sl)];
+        xs_pieces[x_slot(c, j)] = o;
 #pragma unroll
-      for (int i = 0; i < 8; i++) s += (float)v[i];
+        for (int i = 0; i < 8; i++) s += (float)v[i];
+      }
+      xsum[c] = s;
     }
-    xsum[c] = s;
+  } else {
+    // pass 1: val = f16(residual + delta) into LDS (slot order already), sum of squares per thread
+    float ss = 0.f;
+    for (uint32_t c = tid; c < p.nchunks; c += blockDim.x) {
+      const h8* res = reinterpret_cast<const h8*>(x + (size_t)c * 32u);
+      const h8* del = reinterpret_cast<const h8*>(p.delta + (size_t)c * 32u);
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const h8 v = res[j] + del[j];  // f16 addition, as add_norm does
+        h8 o;
+#pragma unroll
+        for (int sl = 0; sl < 8; sl++) o[sl] = v[value_in_slot(sl)];
+        xs_pieces[x_slot(c, j)] = o;
+#pragma unroll
+        for (int i = 0; i < 8; i++) ss = __builtin_fmaf((float)v[i], (float)v[i], ss);
+      }
+    }
+    // the row's sum of squares: lanes by DPP, waves through LDS, every thread adds the wave sums in wave order
+    float* wave_ss = reinterpret_cast<float*>(smem + (size_t)padded_chunks * 68u);
+    ss = group_sum_to_last_lane<64>(ss);
+    if (lane == 63) wave_ss[wave] = ss;
+    __syncthreads();
+    float total = 0.f;
+    for (uint32_t w = 0; w < waves; w++) total += wave_ss[w];
+    const float rms_inv = 1.0f / sqrtf(total / (float)(p.nchunks * 32u) + p.rms_eps);
+    // pass 2: each thread normalises the pieces it wrote (no barrier needed for those), rounding to f16 as the
+    // store of the normed vector did, and sums the rounded values
+    for (uint32_t c = tid; c < p.nchunks; c += blockDim.x) {
+      const h8* gam = reinterpret_cast<const h8*>(p.gamma + (size_t)c * 32u);
+      float s = 0.f;
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const h8 g = gam[j];
+        h8 o = xs_pieces[x_slot(c, j)];
+#pragma unroll
+        for (int sl = 0; sl < 8; sl++) {
+          o[sl] = narrow_f32((float)o[sl] * rms_inv * (float)g[value_in_slot(sl)]);
+          s += (float)o[sl];
+        }
+        xs_pieces[x_slot(c, j)] = o;
+      }
+      xsum[c] = s;
+    }
   }
   // QKV: the rotation of every pair index, once per workgroup, by the threads at the far end of the
   // workgroup (the staging above keeps the first ones busy); cos and sin are long instruction
@@ -331,6 +386,14 @@ hipError_t launch_qkv(const GemvParams& p, int lpr, dim3 grid, uint32_t threads,
 }
 
 template <int BITS, bool AFFINE>
+hipError_t launch_prologue(const GemvParams& p, int lpr, dim3 grid, uint32_t threads, size_t smem, hipStream_t s) {
+  if (lpr == 64) hipLaunchKernelGGL((gemv_kernel<BITS, AFFINE, 64, 1, 512, true, false, true>), grid, dim3(threads), smem, s, p);
+  else if (lpr == 32) hipLaunchKernelGGL((gemv_kernel<BITS, AFFINE, 32, 1, 512, true, false, true>), grid, dim3(threads), smem, s, p);
+  else hipLaunchKernelGGL((gemv_kernel<BITS, AFFINE, 16, 1, 512, true, false, true>), grid, dim3(threads), smem, s, p);
+  return hipGetLastError();
+}
+
+template <int BITS, bool AFFINE>
 hipError_t launch_gated(const GemvParams& p, int lpr, dim3 grid, uint32_t threads, size_t smem, hipStream_t s) {
   if (lpr == 64) hipLaunchKernelGGL((gemv_kernel<BITS, AFFINE, 64, 1, 512, true>), grid, dim3(threads), smem, s, p);
   else if (lpr == 32) hipLaunchKernelGGL((gemv_kernel<BITS, AFFINE, 32, 1, 512, true>), grid, dim3(threads), smem, s, p);
@@ -362,6 +425,7 @@ hipError_t launch_gemv(const MatmulArgs& a, const Tune& t, hipStream_t s) {
   p.in_tok_stride = a.in_tok_stride; p.out_tok_stride = a.out_tok_stride; p.ids_stride = a.ids_stride;
   p.experts = a.experts;
   const bool gated = a.up_weights != nullptr;
+  p.delta = a.delta; p.gamma = a.gamma; p.rms_eps = a.rms_eps;
   p.weights2 = a.up_weights; p.scales2 = a.up_scales; p.biases2 = a.up_biases;
   if (a.qkv) {
     const QkvArgs& q = *a.qkv;
@@ -397,7 +461,8 @@ hipError_t launch_gemv(const MatmulArgs& a, const Tune& t, hipStream_t s) {
   p.ntiles = (a.N + rpw - 1) / rpw;
 
   const uint32_t padded_chunks = (p.nchunks + 63u) & ~63u;
-  const size_t smem = (size_t)padded_chunks * 64 + (size_t)padded_chunks * 4 + (a.qkv ? (size_t)(a.qkv->head_dim / 2) * 8 : 0);
+  const size_t smem = (size_t)padded_chunks * 64 + (size_t)padded_chunks * 4 + (a.qkv ? (size_t)(a.qkv->head_dim / 2) * 8 : 0) +
+                      (a.delta ? 64 : 0);  // the prologue's per-wave sums of squares
 
   const uint32_t wg_tiles = (p.ntiles + waves - 1) / waves;
   gx = gx / pairs;
@@ -410,6 +475,11 @@ hipError_t launch_gemv(const MatmulArgs& a, const Tune& t, hipStream_t s) {
   if (a.qkv) {
     if (a.bits == 4) return a.affine ? launch_qkv<4, true>(p, lpr, grid, threads, smem, s) : launch_qkv<4, false>(p, lpr, grid, threads, smem, s);
     return hipErrorInvalidValue;  // rejected by the entry point
+  }
+  if (gated && a.delta) {
+    if (a.bits == 8 || p.moe) return hipErrorInvalidValue;  // rejected by the entry point
+    if (a.bits == 4) return a.affine ? launch_prologue<4, true>(p, lpr, grid, threads, smem, s) : launch_prologue<4, false>(p, lpr, grid, threads, smem, s);
+    return launch_prologue<3, true>(p, lpr, grid, threads, smem, s);
   }
   if (gated) {
     if (a.bits == 8) return hipErrorInvalidValue;  // rejected by the entry point

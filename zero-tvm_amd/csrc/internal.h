@@ -31,6 +31,10 @@ struct MatmulArgs {
   const uint32_t* up_weights = nullptr;
   const _Float16* up_scales = nullptr;
   const _Float16* up_biases = nullptr;
+  // prologue form of the gated FFN (null = none): `in` is the residual, x = RMSNorm(in + delta) * gamma
+  const _Float16* delta = nullptr;
+  const _Float16* gamma = nullptr;
+  float rms_eps = 0.f;
   const QkvArgs* qkv = nullptr;  // with qkv set, N counts rotary pairs and up_* is the same matrix half a head further
   uint32_t M, N, K, k_packed, spr;
   uint32_t bits, affine, out_f32;

@@ -387,6 +387,31 @@ int ztvm_ffn_gated(ztvm_ctx* ctx, const ztvm_matmul_desc* desc, uint64_t up_weig
   return ZTVM_OK;
 }
 
+int ztvm_ffn_gated_prologue(ztvm_ctx* ctx, const ztvm_matmul_desc* desc, uint64_t up_weights, uint64_t up_scales, uint64_t up_biases,
+                            uint64_t delta, uint64_t gamma, float rms_eps) {
+  if (!ctx) return fail(nullptr, ZTVM_E_INVALID, "null context");
+  char why[256];
+  int rc = validate(desc, why, sizeof why, true);
+  if (rc) return fail(ctx, rc, "ztvm_ffn_gated_prologue: %s", why);
+  if (desc->kernel != ZTVM_KERNEL_AUTO && desc->kernel != ZTVM_KERNEL_GEMV)
+    return fail(ctx, ZTVM_E_UNSUPPORTED, "ztvm_ffn_gated_prologue: kernel: only the GEMV family has the gated form");
+  if (desc->bits == 8) return fail(ctx, ZTVM_E_UNSUPPORTED, "ztvm_ffn_gated_prologue: no 8-bit form");
+  if (desc->slots || desc->M != 1) return fail(ctx, ZTVM_E_UNSUPPORTED, "ztvm_ffn_gated_prologue: one dense activation row (the decode step) only");
+  if (!up_weights || !up_scales || (desc->affine && !up_biases)) return fail(ctx, ZTVM_E_INVALID, "ztvm_ffn_gated_prologue: null up-projection buffer");
+  if ((up_weights | up_scales | up_biases) & 15u) return fail(ctx, ZTVM_E_INVALID, "ztvm_ffn_gated_prologue: up-projection buffers must be 16-byte aligned");
+  if (!delta || !gamma || ((delta | gamma) & 15u)) return fail(ctx, ZTVM_E_INVALID, "ztvm_ffn_gated_prologue: delta and gamma must be given, 16-byte aligned");
+  if (!(rms_eps >= 0.f)) return fail(ctx, ZTVM_E_INVALID, "ztvm_ffn_gated_prologue: rms_eps must be >= 0");
+  MatmulArgs a = to_args(desc);
+  a.up_weights = reinterpret_cast<const uint32_t*>(up_weights);
+  a.up_scales = reinterpret_cast<const _Float16*>(up_scales);
+  a.up_biases = reinterpret_cast<const _Float16*>(up_biases);
+  a.delta = reinterpret_cast<const _Float16*>(delta);
+  a.gamma = reinterpret_cast<const _Float16*>(gamma);
+  a.rms_eps = rms_eps;
+  HIP_TRY(ctx, launch_gemv(a, ctx->tune, ctx->stream));
+  return ZTVM_OK;
+}
+
 // k_slot / v_slot non-zero: the int8-KV-mode variant, K and V go to two [kv_heads*head_dim] scratch rows
 static int qkv_fused_common(ztvm_ctx* ctx, const ztvm_qkv_fused_desc* d, uint64_t k_slot, uint64_t v_slot) {
   const bool scratch = k_slot || v_slot;

@@ -16,7 +16,7 @@ E_INVALID, E_HIP, E_UNSUPPORTED, E_NODEVICE = -1, -2, -3, -4
 EXPORTS = [
     "ztvm_abi_version", "ztvm_last_error", "ztvm_create", "ztvm_destroy", "ztvm_device_info",
     "ztvm_alloc", "ztvm_free", "ztvm_upload", "ztvm_download", "ztvm_fill", "ztvm_copy", "ztvm_sync",
-    "ztvm_matmul_validate", "ztvm_matmul_resolve", "ztvm_matmul", "ztvm_ffn_gated", "ztvm_qkv_fused", "ztvm_qkv_fused_scratch",
+    "ztvm_matmul_validate", "ztvm_matmul_resolve", "ztvm_matmul", "ztvm_ffn_gated", "ztvm_ffn_gated_prologue", "ztvm_qkv_fused", "ztvm_qkv_fused_scratch",
     "ztvm_kv_quantize_int8", "ztvm_dequant",
     "ztvm_record_begin", "ztvm_record_end", "ztvm_submit", "ztvm_cmdbuf_destroy",
     "ztvm_event_create", "ztvm_event_destroy", "ztvm_event_record", "ztvm_event_elapsed_ms",
@@ -99,6 +99,7 @@ def load():
     L.ztvm_get_option.argtypes = [vp, C.c_char_p, C.POINTER(C.c_int)]
     u32, u64 = C.c_uint32, C.c_uint64
     L.ztvm_ffn_gated.argtypes = [vp, C.POINTER(MatmulDesc), u64, u64, u64]
+    L.ztvm_ffn_gated_prologue.argtypes = [vp, C.POINTER(MatmulDesc)] + [C.c_uint64] * 5 + [C.c_float]
     L.ztvm_qkv_fused.argtypes = [vp, C.POINTER(QkvFusedDesc)]
     L.ztvm_qkv_fused_scratch.argtypes = [vp, C.POINTER(QkvFusedDesc), C.c_uint64, C.c_uint64]
     L.ztvm_kv_quantize_int8.argtypes = [vp, C.POINTER(KvQuantizeDesc)]
@@ -195,6 +196,10 @@ class Context:
 
     def ffn_gated(self, desc, up_weights, up_scales, up_biases=0):
         self._chk(self._L.ztvm_ffn_gated(self._h, C.byref(desc), up_weights, up_scales, up_biases))
+
+    def ffn_gated_prologue(self, desc, up_weights, up_scales, up_biases, delta, gamma, rms_eps):
+        self._chk(self._L.ztvm_ffn_gated_prologue(self._h, C.byref(desc), up_weights, up_scales, up_biases, delta, gamma,
+                                                  C.c_float(rms_eps)))
 
     def qkv_fused(self, desc):
         self._chk(self._L.ztvm_qkv_fused(self._h, C.byref(desc)))

@@ -430,6 +430,23 @@ napi_value FfnGated(napi_env env, napi_callback_info info) {  // (ctx, desc, upW
   return rc ? throw_ztvm(env, (ztvm_ctx*)p, rc, "ztvm_ffn_gated") : undefined(env);
 }
 
+napi_value FfnGatedPrologue(napi_env env, napi_callback_info info) {  // (ctx, desc, upWeights, upScales, upBiases, delta, gamma, rmsEps)
+  napi_value a[8];
+  void* p;
+  ztvm_matmul_desc d;
+  uint64_t v[5];
+  double eps = 0;
+  if (!get_args(env, info, 8, a) || !get_ptr(env, a[0], &p) || !get_desc(env, a[1], &d)) return nullptr;
+  for (int i = 0; i < 5; i++)
+    if (!get_u64(env, a[2 + i], &v[i])) return nullptr;
+  if (napi_get_value_double(env, a[7], &eps) != napi_ok) {
+    napi_throw_type_error(env, nullptr, "ztvm addon: rmsEps must be a number");
+    return nullptr;
+  }
+  int rc = ztvm_ffn_gated_prologue((ztvm_ctx*)p, &d, v[0], v[1], v[2], v[3], v[4], (float)eps);
+  return rc ? throw_ztvm(env, (ztvm_ctx*)p, rc, "ztvm_ffn_gated_prologue") : undefined(env);
+}
+
 napi_value RepackPart(napi_env env, napi_callback_info info) {  // (ctx, dst, src, srcBytes, convert, overflow)
   napi_value a[6];
   void* p;
@@ -555,7 +572,7 @@ napi_value Init(napi_env env, napi_value exports) {
       {"validate", Validate}, {"resolve", Resolve}, {"matmul", Matmul}, {"dequant", Dequant}, {"recordBegin", RecordBegin},
       {"recordEnd", RecordEnd}, {"submit", Submit}, {"cmdbufDestroy", CmdbufDestroy}, {"setOption", SetOption},
       {"siluMul", SiluMul}, {"moeCombine", MoeCombine}, {"moeRouterLogits", MoeRouterLogits}, {"moeRouterTopk", MoeRouterTopk},
-      {"moeSlotTranslate", MoeSlotTranslate}, {"ffnGated", FfnGated}, {"repackPart", RepackPart},
+      {"moeSlotTranslate", MoeSlotTranslate}, {"ffnGated", FfnGated}, {"ffnGatedPrologue", FfnGatedPrologue}, {"repackPart", RepackPart},
       {"repackPermuteRows", RepackPermuteRows}, {"repackDequantSplit", RepackDequantSplit}, {"qkvFused", QkvFused},
       {"qkvFusedScratch", QkvFusedScratch}, {"kvQuantizeInt8", KvQuantizeInt8}};
   for (const E& e : table) {

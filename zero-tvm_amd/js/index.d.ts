@@ -39,6 +39,8 @@ export declare class Device {
   moeSlotTranslate(idsOut: BindEntry, idsIn: BindEntry, slotMap: BindEntry, n: number, mapLen: number): void
   ffnGated(pipeline: Pipeline, group: BindGroup, upWeights: BindEntry, upScales: BindEntry, upBiases: BindEntry | null,
     wgX?: number, wgY?: number, wgZ?: number): void
+  ffnGatedPrologue(pipeline: Pipeline, group: BindGroup, upWeights: BindEntry, upScales: BindEntry, upBiases: BindEntry | null,
+    delta: BindEntry, gamma: BindEntry, rmsEps: number, wgX?: number, wgY?: number, wgZ?: number): void
   qkvFused(bufs: BindEntry[], pod: Uniform, model: { d: number; affine?: boolean; heads: number; kvHeads: number; headDim: number
     pageSize: number; kvPageStride: number; headPageStride: number; vPageOffset: number; ropeTheta: number }): void
   qkvFusedScratch(bufs: BindEntry[], pod: Uniform, model: { d: number; affine?: boolean; heads: number; kvHeads: number

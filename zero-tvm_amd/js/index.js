@@ -266,6 +266,15 @@ class Device {
     addon().ffnGated(this.ctx, this.descriptor(group, wgX, wgY, wgZ), this._a(upWeights), this._a(upScales), this._a(upBiases))
   }
   /**
+   * fused_ffn_prologue.wgsl: ffnGated with the FFN-entry add + RMSNorm folded in; the bind group's input (binding 1)
+   * is the residual, `delta` the o-proj output added to it, `gamma` the norm gain, rmsEps the prelude's RMS_EPS
+   */
+  ffnGatedPrologue(pipeline, group, upWeights, upScales, upBiases, delta, gamma, rmsEps, wgX, wgY, wgZ) {
+    if (group.pipeline !== pipeline) throw new Error("ffnGatedPrologue: bind group was built for '" + group.pipeline.label + "', not '" + pipeline.label + "'")
+    addon().ffnGatedPrologue(this.ctx, this.descriptor(group, wgX, wgY, wgZ), this._a(upWeights), this._a(upScales), this._a(upBiases),
+      this._a(delta), this._a(gamma), rmsEps)
+  }
+  /**
    * qkv_fused*.wgsl: bindings [q_out, kv_pages, hidden, scales, weights, position_map, (biases)], the PODArgs
    * {position_map_elem_offset, pages_elem_offset} and the model constants of the shader prelude
    * (heads, kvHeads, headDim, pageSize, kvPageStride, headPageStride, vPageOffset, ropeTheta).
