@@ -182,36 +182,40 @@ __global__ __launch_bounds__(256) void router_logits_kernel(float* __restrict__ 
 // (src/compiler/shaders/moe_router_topk.wgsl:67-136). One wave per token; lane l
 // holds experts l, l+64, ... (coalesced reads); nothing leaves registers.
 //
-// The K arg-max rounds are a serial chain, so each round is kept short: a probability and
-// its expert travel as ONE 64-bit key (f32 bits of the probability, which order like the
-// value for non-negative floats, above the complemented index, so the larger key is the
-// larger probability and, among equals, the lower index), and the wave-wide maximum is a
-// six-step scan over data-parallel-primitive moves instead of cross-lane LDS permutes.
+// The K arg-max rounds are a serial chain, so each round is kept short: two six-step scans over
+// data-parallel-primitive moves on 32-bit values (the largest probability, then the lowest index
+// holding it) instead of cross-lane LDS permutes or 64-bit keys, and only as many registers per
+// lane as the expert count needs.
 constexpr int TOPK_PER = 8;  // 64 lanes x 8 = 512 experts at most
 
-__device__ __forceinline__ uint64_t key_max(uint64_t a, uint64_t b) { return a > b ? a : b; }
-
 template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ uint64_t dpp_max(uint64_t v) {
-  // lanes without a source (and rows outside ROW_MASK) take 0, the identity of max over keys
-  const uint32_t lo = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)v, CTRL, ROW_MASK, 0xF, false);
-  const uint32_t hi = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)(v >> 32), CTRL, ROW_MASK, 0xF, false);
-  return key_max(v, ((uint64_t)hi << 32) | lo);
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t v, uint32_t identity) {
+  return (uint32_t)__builtin_amdgcn_update_dpp((int)identity, (int)v, CTRL, ROW_MASK, 0xF, false);
+}
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+  v = max(v, dpp_u32<0x111, 0xF>(v, 0u));
+  v = max(v, dpp_u32<0x112, 0xF>(v, 0u));
+  v = max(v, dpp_u32<0x114, 0xF>(v, 0u));
+  v = max(v, dpp_u32<0x118, 0xF>(v, 0u));
+  v = max(v, dpp_u32<0x142, 0xA>(v, 0u));
+  v = max(v, dpp_u32<0x143, 0xC>(v, 0u));
+  return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
+}
+__device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) {
+  v = min(v, dpp_u32<0x111, 0xF>(v, ~0u));
+  v = min(v, dpp_u32<0x112, 0xF>(v, ~0u));
+  v = min(v, dpp_u32<0x114, 0xF>(v, ~0u));
+  v = min(v, dpp_u32<0x118, 0xF>(v, ~0u));
+  v = min(v, dpp_u32<0x142, 0xA>(v, ~0u));
+  v = min(v, dpp_u32<0x143, 0xC>(v, ~0u));
+  return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
 }
 
-// maximum of v over the 64 lanes, returned to every lane
-__device__ __forceinline__ uint64_t wave_key_max(uint64_t v) {
-  v = dpp_max<0x111, 0xF>(v);  // row_shr:1
-  v = dpp_max<0x112, 0xF>(v);  // row_shr:2
-  v = dpp_max<0x114, 0xF>(v);  // row_shr:4
-  v = dpp_max<0x118, 0xF>(v);  // row_shr:8   -> lane 15 of each row holds the row's maximum
-  v = dpp_max<0x142, 0xA>(v);  // row_bcast:15 into rows 1 and 3
-  v = dpp_max<0x143, 0xC>(v);  // row_bcast:31 into rows 2 and 3 -> lane 63 holds the wave's maximum
-  const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, 63);
-  const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), 63);
-  return ((uint64_t)hi << 32) | lo;
-}
-
+// PER = experts per lane (E <= 64 * PER). A candidate is the bit pattern of its probability plus one
+// (probabilities are non-negative floats, so their bit patterns order like the values; zero marks
+// "none" and "already taken", and an underflowed probability of exactly 0 is still a candidate). Each
+// of the K rounds takes the wave's largest candidate, then the lowest expert index holding it.
+template <int PER>
 __global__ __launch_bounds__(256) void router_topk_kernel(uint32_t* __restrict__ out_idx, float* __restrict__ out_score,
                                                           const float* __restrict__ logits, uint32_t E, uint32_t K,
                                                           uint32_t norm_topk, uint32_t has_shared, uint32_t tokens) {
@@ -221,10 +225,10 @@ __global__ __launch_bounds__(256) void router_topk_kernel(uint32_t* __restrict__
   const float* l = logits + (size_t)tok * (E + has_shared);
   const size_t obase = (size_t)tok * (K + has_shared);
 
-  float pv[TOPK_PER];
+  float pv[PER];
   float m = -3.0e38f;
 #pragma unroll
-  for (int i = 0; i < TOPK_PER; i++) {
+  for (int i = 0; i < PER; i++) {
     const uint32_t e = lane + 64u * i;
     pv[i] = e < E ? l[e] : -3.0e38f;
     m = fmaxf(m, pv[i]);
@@ -232,33 +236,36 @@ __global__ __launch_bounds__(256) void router_topk_kernel(uint32_t* __restrict__
   const float shared_logit = has_shared ? l[E] : 0.f;
   const float peak = wave_max(m);
   float s = 0.f;
-  // key 0 = "no candidate": every real candidate carries a non-zero complemented index
-  uint64_t key[TOPK_PER];
+  uint32_t cand[PER];
 #pragma unroll
-  for (int i = 0; i < TOPK_PER; i++) {
+  for (int i = 0; i < PER; i++) {
     const uint32_t e = lane + 64u * i;
     const float p = e < E ? expf(pv[i] - peak) : 0.f;
     s += p;
-    key[i] = e < E ? ((uint64_t)__builtin_bit_cast(uint32_t, p) << 32) | (0xffffffffu - e) : 0ull;
+    cand[i] = e < E ? __builtin_bit_cast(uint32_t, p) + 1u : 0u;
   }
   const float denom = wave_sum(s);
 
   float total = 0.f, mine = 0.f;
   uint32_t mine_idx = 0;
   for (uint32_t k = 0; k < K; k++) {
-    uint64_t best = key[0];
+    uint32_t best = cand[0];
 #pragma unroll
-    for (int i = 1; i < TOPK_PER; i++) best = key_max(best, key[i]);
-    best = wave_key_max(best);
-    const float bv = __builtin_bit_cast(float, (uint32_t)(best >> 32));
+    for (int i = 1; i < PER; i++) best = max(best, cand[i]);
+    best = wave_max_u32(best);
+    uint32_t holder = ~0u;  // this lane's lowest expert index holding `best`
+#pragma unroll
+    for (int i = PER - 1; i >= 0; i--) holder = cand[i] == best ? lane + 64u * i : holder;
+    const uint32_t win = wave_min_u32(holder);
+    const float bv = __builtin_bit_cast(float, best - 1u);
     total += bv;
     if (lane == k) {
       mine = bv;
-      mine_idx = 0xffffffffu - (uint32_t)best;
+      mine_idx = win;
     }
 #pragma unroll
-    for (int i = 0; i < TOPK_PER; i++)
-      if (key[i] == best) key[i] = 0ull;  // keys are unique: exactly one register of one lane
+    for (int i = 0; i < PER; i++)
+      if (lane + 64u * i == win) cand[i] = 0u;
   }
   const float scale = norm_topk ? 1.0f / total : 1.0f / denom;
   if (lane < K) {
@@ -401,9 +408,14 @@ uint32_t router_topk_max_experts() { return 64u * TOPK_PER; }
 
 hipError_t launch_router_topk(void* out_idx, void* out_score, const void* logits, uint32_t E, uint32_t K, uint32_t norm_topk,
                               uint32_t has_shared, uint32_t tokens, hipStream_t s) {
-  hipLaunchKernelGGL(router_topk_kernel, dim3((tokens + 3) / 4), dim3(256), 0, s, reinterpret_cast<uint32_t*>(out_idx),
-                     reinterpret_cast<float*>(out_score), reinterpret_cast<const float*>(logits), E, K, norm_topk, has_shared,
-                     tokens);
+  auto go = [&](auto k) {
+    hipLaunchKernelGGL(k, dim3((tokens + 3) / 4), dim3(256), 0, s, reinterpret_cast<uint32_t*>(out_idx),
+                       reinterpret_cast<float*>(out_score), reinterpret_cast<const float*>(logits), E, K, norm_topk, has_shared, tokens);
+  };
+  if (E <= 64) go(router_topk_kernel<1>);
+  else if (E <= 128) go(router_topk_kernel<2>);
+  else if (E <= 256) go(router_topk_kernel<4>);
+  else go(router_topk_kernel<TOPK_PER>);
   return hipGetLastError();
 }
 
