@@ -142,6 +142,11 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(const GemvParams p) {
   UnpackConsts kc;
   kc.init();
 
+  // QKV: the token's position, fetched now (a uniform load) so that neither the rotary table nor the
+  // scatter at the end of a row waits for it
+  int position = 0;
+  if (QKV) position = p.position_map[p.pos_off];
+
   // Loads of one (tile, pass), as buffer loads: a uniform descriptor (this expert's matrix) plus one
   // 32-bit byte offset per lane, and an offset past the end of the array returns zeros without
   // touching memory. Rows past N are past the end by themselves (so are whole tiles past the last
@@ -267,8 +272,14 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(const GemvParams p) {
   if (QKV) {
     const uint32_t rt = blockDim.x - 1u - tid;
     if (rt < p.half_dim) {
-      const float freq = (float)p.position_map[p.pos_off] / powf(p.rope_theta, (float)(rt * 2u) / (float)p.head_dim);
-      rope[rt] = float2{cosf(freq), sinf(freq)};
+      const float freq = (float)position / powf(p.rope_theta, (float)(rt * 2u) / (float)p.head_dim);
+      // the hardware sine and cosine take revolutions and are accurate to about 1e-6 on [0, 1): turning the
+      // angle into a fraction of a revolution costs it about |freq| * 2^-24, below what forming the f32
+      // angle itself already carries (position * 2^-23), and replaces two long range reductions that
+      // every wave of the workgroup would wait for at the barrier
+      const float turns = freq * 0.15915494309189535f;
+      const float frac = turns - floorf(turns);
+      rope[rt] = float2{__builtin_amdgcn_cosf(frac), __builtin_amdgcn_sinf(frac)};
     }
   }
   __syncthreads();
@@ -333,7 +344,6 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(const GemvParams p) {
         if (QKV) {
           if (lk == LPR - 1 && rr < p.N) {
             const QkvPair q = qkv_pair(p, rr);
-            const int position = p.position_map[p.pos_off];
             const uint32_t page_no = (uint32_t)position / p.page_size, slot = (uint32_t)position - page_no * p.page_size;
             const size_t cache = (size_t)page_no * p.kv_page_stride + (size_t)q.head * p.head_page_stride +
                                  (size_t)slot * p.head_dim + p.pages_off + q.dim_lo;
