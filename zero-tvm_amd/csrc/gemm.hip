@@ -33,7 +33,11 @@
 //              step s+2 are unpacked from registers into the same stage, the
 //              fragments of step s+1 are read while those of step s retire,
 //              and the previous run's partial sums are folded between MFMAs;
-//              one barrier per step
+//              one barrier per step. Every matrix instruction is followed by
+//              its share of that other work (about seven vector instructions
+//              fit in the 32 cycles one of them occupies the matrix core)
+//   scales     fetched six steps at a time, global -> LDS like the activations,
+//              into a two-batch ring, as stored (f16)
 //   grid       one workgroup per tile, ids remapped so that the tiles sharing
 //              a weight panel run on the same XCD (same L2)
 #include "internal.h"
@@ -117,6 +121,40 @@ __device__ __forceinline__ void static_for(F&& f) {
 }
 
 constexpr int NSTAGE = 3;
+constexpr int SCB = 6;  // steps per batch of scales: two turns of the three LDS stages, so the hot loop has no branch
+
+// 16 bytes per lane from global memory (uniform base + 32-bit lane offset) straight into LDS slot
+// lds + 16 * lane. Written as assembly: the compiler's wait-count pass treats the builtin as an
+// access to both vector memory and LDS, and while one is pending it turns every later LDS wait
+// into a full drain. The loads are counted by vmcnt like any other; the kernel waits for them
+// itself (vmcnt(0) before the barrier that ends a step). M0 carries the LDS address; nothing
+// else in these kernels uses M0.
+__device__ __forceinline__ void dma16(const void* base_uniform, uint32_t off, uint32_t lds_uniform) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base_uniform), "s"(lds_uniform)
+               : "memory");
+}
+// The same with 4 bytes per lane: LDS slot lds + 4 * lane.
+__device__ __forceinline__ void dma4(const void* base_uniform, uint32_t off, uint32_t lds_uniform) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(off), "s"(base_uniform), "s"(lds_uniform) : "memory");
+}
+
+// Work that shares a step with the 16 matrix instructions, by half-slot hs = 2 * pair + (0 after
+// the first MFMA of the pair, 1 after the second). The thread's packed words are unpacked in the
+// first eight half-slots, evenly spaced; the 32 fold FMAs of a run are spread over the run's
+// half-slots that have no unpack (over all of them when every one has).
+template <int W_WORDS>
+constexpr bool has_unpack(int hs) { return hs < 8 && hs % (8 / W_WORDS) == 0; }
+template <int W_WORDS, int RUNH>
+constexpr int fold_upto(int hs) {  // FMAs of the run done before half-slot hs
+  const int r0 = hs / RUNH * RUNH;
+  int total = 0;
+  for (int k = r0; k < r0 + RUNH; k++) total += has_unpack<W_WORDS>(k) ? 0 : 1;
+  const bool flat = total == 0;
+  if (flat) total = RUNH;
+  int before = 0;
+  for (int k = r0; k < hs; k++) before += flat ? 1 : (has_unpack<W_WORDS>(k) ? 0 : 1);
+  return 32 * before / total;
+}
 
 // The 16 MFMAs of a step as 8 pairs (block row i, k slice ks) x 2 block columns. A run of pairs
 // accumulates one group into one partial set (set = i); affine: 64-k groups, runs of 4 pairs;
@@ -139,16 +177,18 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
   static_assert(A_LOADS >= 1 && (W_WORDS == 2 || W_WORDS == 4 || W_WORDS == 8), "tile/thread mismatch");
   constexpr int W_TPR = 8 / W_WORDS;              // threads per weight row
   constexpr int SCALES = AFFINE ? 1 : 2;          // groups per step
-  constexpr int SC_LOADS = (TN * SCALES + THREADS - 1) / THREADS;
   constexpr uint32_t ROW_BYTES = CHUNKS * 16;
   constexpr uint32_t STAGE_BYTES = (TM + TN) * ROW_BYTES;
   constexpr uint32_t W_BASE = TM * ROW_BYTES;          // weight rows follow the activation rows of a stage
-  constexpr uint32_t SC_BASE = NSTAGE * STAGE_BYTES;   // float [NSTAGE][TN][SCALES]
-  constexpr uint32_t SC_STAGE = TN * SCALES * 4;
+  constexpr uint32_t SC_BASE = NSTAGE * STAGE_BYTES;   // f16 [2 batches][SC_PAIRS][TN][2]
+  constexpr int SC_PAIRS = SCB * SCALES / 2;           // 4-byte pairs per column per batch
+  constexpr uint32_t SC_BATCH = SC_PAIRS * TN * 4;
+  static_assert(TN % 64 == 0 && TN <= THREADS, "whole waves load the scales");
 
   extern __shared__ __align__(16) unsigned char smem[];
 
   const uint32_t tid = threadIdx.x, lane = tid & 63u;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(lptr_t)smem;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const uint32_t wm = wave / WN, wn = wave % WN;
 
@@ -166,76 +206,75 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
   // ---- activations: global -> LDS without passing registers. One instruction fills 64
   // consecutive 16-byte LDS slots (8 rows), slot = lane; the lane fetches the chunk that the
   // swizzle places there. Rows past M repeat row M-1: they are computed and never stored.
-  const _Float16* a_src[A_LOADS];
-  const _Float16* xs_src[A_LOADS];
+  // Instruction i of a wave fills the eight tile rows of group i * WAVES + wave. A group reaching
+  // past row M is moved back to end at row M - 1 (with M < 8: to row 0, and the lanes clamp), so
+  // that one lane offset serves every group and the group's base stays uniform. Its tile rows
+  // then repeat rows of the group before; the stores at the end use the same mapping.
+  static_assert(WAVES % 2 == 0, "the swizzle of a lane's row must not depend on the instruction");
+  const uint32_t lrow = lane >> 3;
+  const uint32_t a_ch = (lane & 7u) ^ swz(wave * 8 + lrow);
+  const uint32_t lrow_c = lrow < p.M ? lrow : p.M - 1;
+  const uint32_t a_lane = (lrow_c * p.K + a_ch * 8) * 2u;
+  const uint32_t xs_lane = (lrow_c * p.xs_stride + a_ch * 8) * 2u;
+  uint32_t a_row0[A_LOADS];
 #pragma unroll
   for (int i = 0; i < A_LOADS; i++) {
-    const uint32_t row = (i * WAVES + wave) * 8 + (lane >> 3);
-    const uint32_t ch = (lane & 7u) ^ swz(row);
-    uint32_t m = m0 + row;
-    m = m < p.M ? m : p.M - 1;
-    a_src[i] = p.in + (size_t)m * p.K + ch * 8;
-    xs_src[i] = p.xs16 + (size_t)m * p.xs_stride + ch * 8;
+    const uint32_t row0 = m0 + (i * WAVES + wave) * 8, last = p.M >= 8 ? p.M - 8 : 0;
+    a_row0[i] = row0 < last ? row0 : last;
   }
-  auto load_a = [&](const _Float16** src, uint32_t stage) __attribute__((always_inline)) {
+  const _Float16* a_base[A_LOADS];  // uniform; move one k step per fill
 #pragma unroll
-    for (int i = 0; i < A_LOADS; i++) {
-      __builtin_amdgcn_global_load_lds((gptr_t)src[i], (lptr_t)(smem + stage * STAGE_BYTES + (i * WAVES + wave) * 1024u), 16, 0, 0);
-      src[i] += KS;
-    }
-  };
+  for (int i = 0; i < A_LOADS; i++) a_base[i] = p.in + (size_t)a_row0[i] * p.K;
+  auto lds_slot = [&](uint32_t stage, int i) __attribute__((always_inline)) { return lds0 + stage * STAGE_BYTES + (i * WAVES + wave) * 1024u; };
 
   // ---- weights: registers, unpack, LDS
   const uint32_t w_row = tid / W_TPR, w_part = tid % W_TPR;
   uint32_t w_n = n0 + w_row;
   w_n = w_n < p.N ? w_n : p.N - 1;  // clamped rows are never stored
-  const uint32_t* w_src = p.weights + (size_t)w_n * p.k_packed + w_part * W_WORDS;
+  // one descriptor + 32-bit lane offset + uniform step offset: no address arithmetic in the loop
+  const __amdgpu_buffer_rsrc_t wres = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(p.weights), 0, p.N * p.k_packed * 4u, 0x00020000);
+  const uint32_t w_off = (w_n * p.k_packed + w_part * W_WORDS) * 4u;
+  uint32_t w_adv = 0;  // uniform, bytes
   uint32_t w_dst[W_WORDS];
 #pragma unroll
   for (int j = 0; j < W_WORDS; j++) w_dst[j] = W_BASE + w_row * ROW_BYTES + (((w_part * W_WORDS + j) ^ swz(w_row)) << 4);
-  // scales: thread -> (column, group of the step); surplus threads repeat the last one
-  const _Float16* sc_src[SC_LOADS];
-  uint32_t sc_dst[SC_LOADS];
-#pragma unroll
-  for (int i = 0; i < SC_LOADS; i++) {
-    uint32_t idx = tid + i * THREADS;
-    idx = idx < TN * SCALES ? idx : TN * SCALES - 1;
-    uint32_t n = n0 + idx / SCALES;
-    n = n < p.N ? n : p.N - 1;
-    sc_src[i] = p.scales + (size_t)n * p.spr + idx % SCALES;
-    sc_dst[i] = SC_BASE + idx * 4;
-  }
 
   struct WRegs {
     uint32_t w[W_WORDS];
-    _Float16 s[SC_LOADS];
   };
   auto load_w = [&](WRegs& r) __attribute__((always_inline)) {
     if (W_WORDS == 2) {
-      const u32x2 v = *reinterpret_cast<const u32x2*>(w_src);
+      const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(wres, w_off, w_adv, 0);
       r.w[0] = v.x; r.w[1] = v.y;
     } else {
 #pragma unroll
       for (int q4 = 0; q4 < W_WORDS / 4; q4++) {
-        const u32x4 v = *reinterpret_cast<const u32x4*>(w_src + 4 * q4);
+        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(wres, w_off + 16 * q4, w_adv, 0);
         r.w[4 * q4 + 0] = v.x; r.w[4 * q4 + 1] = v.y; r.w[4 * q4 + 2] = v.z; r.w[4 * q4 + 3] = v.w;
       }
     }
-#pragma unroll
-    for (int i = 0; i < SC_LOADS; i++) {
-      r.s[i] = *sc_src[i];
-      sc_src[i] += SCALES;
-    }
-    w_src += KS / 8;
+    w_adv += KS / 2;
   };
   auto store_w_words = [&](const WRegs& r, uint32_t stage, int j0, int j1) __attribute__((always_inline)) {
 #pragma unroll
     for (int j = j0; j < j1; j++)
       *reinterpret_cast<h8*>(smem + stage * STAGE_BYTES + w_dst[j]) = unpack_word_natural<AFFINE>(r.w[j], c_mixed);
   };
-  auto store_w_scales = [&](const WRegs& r, uint32_t stage) __attribute__((always_inline)) {
+
+  // ---- scales: the first TN / 64 waves fetch SCB steps of their 64 columns at a time, one pair
+  // of f16 (4 bytes) per lane and instruction, into batch slot (batch & 1) of the ring, laid out
+  // [pair][column]. Pairs past a row's end repeat the row's last pair and are never used.
+  const bool sc_loader = wave < TN / 64;
+  uint32_t sc_n = n0 + tid;
+  sc_n = sc_n < p.N ? sc_n : p.N - 1;
+  const uint32_t sc_off = sc_n * p.spr * 2u;  // spr is even (checked on the host): rows start on 4 bytes
+  auto load_sc = [&](uint32_t batch) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < SC_LOADS; i++) *reinterpret_cast<float*>(smem + stage * SC_STAGE + sc_dst[i]) = (float)r.s[i];
+    for (int k = 0; k < SC_PAIRS; k++) {
+      uint32_t e = batch * (SCB * SCALES) + 2 * k;
+      e = e < p.spr - 2 ? e : p.spr - 2;
+      dma4(p.scales, sc_off + e * 2u, lds0 + SC_BASE + (batch & 1u) * SC_BATCH + k * (TN * 4) + wave * 256u);
+    }
   };
 
   // ---- operand fragments: lane -> row frow of a 32-row block, k slice fk of the 16
@@ -247,7 +286,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
     a_rd[ks] = x + wm * 64 * ROW_BYTES;
     b_rd[ks] = x + W_BASE + wn * 64 * ROW_BYTES;
   }
-  const uint32_t sc_rd = SC_BASE + (wn * 64 + frow) * SCALES * 4;
+  const uint32_t sc_rd = SC_BASE + (wn * 64 + frow) * 4;
   auto read_a = [&](uint32_t stage, int i, int ks) __attribute__((always_inline)) {
     return *reinterpret_cast<const h8*>(smem + stage * STAGE_BYTES + a_rd[ks] + i * 32 * ROW_BYTES);
   };
@@ -270,7 +309,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
     const uint32_t G = p.spr;
     const _Float16* brow = p.biases + (size_t)w_n * G;
     for (uint32_t bs = 0; bs < p.bias_steps; bs++) {
-      load_a(xs_src, 0);
+#pragma unroll
+      for (int i = 0; i < A_LOADS; i++) dma16(p.xs16 + (size_t)a_row0[i] * p.xs_stride + bs * KS, xs_lane, lds_slot(0, i));
 #pragma unroll
       for (int j = 0; j < W_WORDS; j++) {
         const uint32_t col = bs * KS + (w_part * W_WORDS + j) * 8;  // column c meets b[n][c mod G]; zero past 2G
@@ -316,16 +356,22 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
   WRegs wcur, wnext;
 
   const uint32_t nsteps = p.nsteps;
-  // prologue: stages 0 and 1 complete, weights of step 2 in registers
-  load_a(a_src, 0);
+  // prologue: stages 0 and 1 complete, weights of step 2 in registers, scale batch 0 in the ring
+  if (sc_loader) load_sc(0);
+  auto load_a = [&](uint32_t stage) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < A_LOADS; i++) {
+      dma16(a_base[i], a_lane, lds_slot(stage, i));
+      a_base[i] += KS;
+    }
+  };
+  load_a(0);
   load_w(wcur);
   store_w_words(wcur, 0, 0, W_WORDS);
-  store_w_scales(wcur, 0);
   if (nsteps > 1) {
-    load_a(a_src, 1);
+    load_a(1);
     load_w(wcur);
     store_w_words(wcur, 1, 0, W_WORDS);
-    store_w_scales(wcur, 1);
   }
   if (nsteps > 2) load_w(wcur);
   __builtin_amdgcn_s_waitcnt(0x0070);
@@ -349,58 +395,73 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
     for (int g = 0; g < SCALES; g++) sc[g][j] = 0.f;
   }
 
-  auto step = [&](auto hot_c, uint32_t cur, uint32_t nxt, uint32_t fill, bool fetch_a, bool fetch_w) __attribute__((always_inline)) {
+  // pos: place of the step in its batch of scales, batch: that batch, fetch_sc: fetch the next one
+  auto step = [&](auto hot_c, uint32_t cur, uint32_t nxt, uint32_t fill, bool fetch_a, bool fetch_w, uint32_t pos, uint32_t batch,
+                  bool fetch_sc) __attribute__((always_inline)) {
     constexpr bool HOT = decltype(hot_c)::value;
+    constexpr int RUNH = 2 * S::RUN;
     if (HOT || fetch_w) load_w(wnext);
+    // the next batch of scales is fetched in the first step of a batch (its ring slot was last
+    // read a step ago) and first read six steps on
+    if (fetch_sc && sc_loader) load_sc(batch + 1);
+    {
+      const uint32_t e = pos * SCALES;  // element of the batch: pair e / 2, half e % 2
+      const uint32_t at = sc_rd + (batch & 1u) * SC_BATCH + (e >> 1) * (TN * 4) + (e & 1u) * 2;
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-      scp[j] = sc[SCALES - 1][j];
+      for (int j = 0; j < 2; j++) {
+        scp[j] = sc[SCALES - 1][j];
 #pragma unroll
-      for (int g = 0; g < SCALES; g++)
-        sc[g][j] = *reinterpret_cast<const float*>(smem + cur * SC_STAGE + sc_rd + (j * 32 * SCALES + g) * 4);
+        for (int g = 0; g < SCALES; g++) sc[g][j] = (float)*reinterpret_cast<const _Float16*>(smem + at + j * 32 * 4 + g * 2);
+      }
     }
     static_for<8>([&](auto pc) {
       constexpr int pp = decltype(pc)::value;
       constexpr int i = S::I(pp), ks = S::KSL(pp);
       constexpr bool first = pp % S::RUN == 0;
+      // the run that ended before this one is folded into the totals: tot += scale * part
+      constexpr int prev = (pp - pp % S::RUN + 8 - S::RUN) % 8;  // first pair of the previous run
+      constexpr int fi = S::I(prev), fg = S::GRP(prev);
+      constexpr bool from_last_step = pp < S::RUN;
+      auto fold = [&](auto hs_c) __attribute__((always_inline)) {
+        constexpr int hs = decltype(hs_c)::value;
+        constexpr int q0 = fold_upto<W_WORDS, RUNH>(hs), q1 = (hs + 1) % RUNH == 0 ? 32 : fold_upto<W_WORDS, RUNH>(hs + 1);
 #pragma unroll
-      for (int j = 0; j < 2; j++)
-        part[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(Aq[pp % 4], Bf[j][ks], first ? zero : part[i][j], 0, 0, 0);
+        for (int q = q0; q < q1; q++) {
+          const int j = q / 16, e = q % 16;
+          const float sv = from_last_step ? scp[j] : sc[fg][j];
+          tot[fi][j][e] = __builtin_fmaf(sv, part[fi][j][e], tot[fi][j][e]);
+        }
+      };
+      auto unpack = [&](auto hs_c) __attribute__((always_inline)) {
+        constexpr int hs = decltype(hs_c)::value;
+        if constexpr (has_unpack<W_WORDS>(hs)) {
+          constexpr int j = hs / (8 / W_WORDS);
+          if (HOT || fetch_a) store_w_words(wcur, fill, j, j + 1);
+        }
+      };
+      using hs0 = std::integral_constant<int, 2 * pp>;
+      using hs1 = std::integral_constant<int, 2 * pp + 1>;
+      part[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(Aq[pp % 4], Bf[0][ks], first ? zero : part[i][0], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
-      // the fragment slot just used takes the pair four places on; after block row 1 the
-      // weight fragments of this k slice are done and the next step's replace them
+      // after block row 1 the weight fragments of this k slice are done: the next step's replace them
+      if (i == 1) Bf[0][ks] = read_b(nxt, 0, ks);
+      fold(hs0{});
+      unpack(hs0{});
+      __builtin_amdgcn_sched_barrier(0);
+      part[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(Aq[pp % 4], Bf[1][ks], first ? zero : part[i][1], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      // the activation fragment slot just used takes the pair four places on
       if (pp + 4 < 8) Aq[pp % 4] = read_a(cur, S::I(pp + 4), S::KSL(pp + 4));
       else Aq[pp % 4] = read_a(nxt, S::I(pp - 4), S::KSL(pp - 4));
-      if (i == 1) {
-#pragma unroll
-        for (int j = 0; j < 2; j++) Bf[j][ks] = read_b(nxt, j, ks);
-      }
-      // fold a slice of the run that ended before this one: tot += scale * part
-      {
-        constexpr int prev = (pp - pp % S::RUN + 8 - S::RUN) % 8;      // first pair of the previous run
-        constexpr int fi = S::I(prev), fg = S::GRP(prev);
-        constexpr bool from_last_step = pp < S::RUN;
-        constexpr int per = 32 / S::RUN, lo = (pp % S::RUN) * per;     // 32 FMAs per run of 2 blocks
-#pragma unroll
-        for (int q = lo; q < lo + per; q++) {
-          const int j = q / 16, e = q % 16;
-          const float s = from_last_step ? scp[j] : sc[fg][j];
-          tot[fi][j][e] = __builtin_fmaf(s, part[fi][j][e], tot[fi][j][e]);
-        }
-      }
+      if (i == 1) Bf[1][ks] = read_b(nxt, 1, ks);
+      fold(hs1{});
+      unpack(hs1{});
       if (HOT || fetch_a) {
         constexpr int i0 = pp * A_LOADS / 4, i1 = (pp + 1) * A_LOADS / 4;  // spread over the first four pairs
 #pragma unroll
         for (int ia = i0; ia < i1 && ia < A_LOADS; ia++) {
-          __builtin_amdgcn_global_load_lds((gptr_t)a_src[ia], (lptr_t)(smem + fill * STAGE_BYTES + (ia * WAVES + wave) * 1024u), 16, 0, 0);
-          a_src[ia] += KS;
-        }
-      }
-      if (HOT || fetch_a) {
-        if (pp == 0) store_w_words(wcur, fill, 0, W_WORDS / 2);
-        if (pp == 1) {
-          store_w_words(wcur, fill, W_WORDS / 2, W_WORDS);
-          store_w_scales(wcur, fill);
+          dma16(a_base[ia], a_lane, lds_slot(fill, ia));
+          a_base[ia] += KS;
         }
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -416,14 +477,20 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
 
   using hot_t = std::integral_constant<bool, true>;
   using cold_t = std::integral_constant<bool, false>;
-  uint32_t s = 0;
-  // hot: steps whose s+3 is still a main step
-  for (; s + 6 <= nsteps; s += 3) {
-    step(hot_t{}, 0, 1, 2, true, true);
-    step(hot_t{}, 1, 2, 0, true, true);
-    step(hot_t{}, 2, 0, 1, true, true);
+  uint32_t s = 0, batch = 0;
+  // hot: one batch of scales per turn; every step's s+3 is still a main step
+  for (; s + SCB + 3 <= nsteps; s += SCB, batch++) {
+    step(hot_t{}, 0, 1, 2, true, true, 0, batch, true);
+    step(hot_t{}, 1, 2, 0, true, true, 1, batch, false);
+    step(hot_t{}, 2, 0, 1, true, true, 2, batch, false);
+    step(hot_t{}, 0, 1, 2, true, true, 3, batch, false);
+    step(hot_t{}, 1, 2, 0, true, true, 4, batch, false);
+    step(hot_t{}, 2, 0, 1, true, true, 5, batch, false);
   }
-  for (; s < nsteps; s++) step(cold_t{}, s % 3, (s + 1) % 3, (s + 2) % 3, s + 2 < nsteps, s + 3 < nsteps);
+  for (uint32_t pos = 0; s < nsteps; s++) {
+    step(cold_t{}, s % 3, (s + 1) % 3, (s + 2) % 3, s + 2 < nsteps, s + 3 < nsteps, pos, batch, pos == 0 && s + SCB < nsteps);
+    if (++pos == SCB) pos = 0, batch++;
+  }
   // the last run of the last step is still unfolded
 #pragma unroll
   for (int j = 0; j < 2; j++)
@@ -438,8 +505,11 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
       const uint32_t n = n0 + wn * 64 + j * 32 + (lane & 31u);
 #pragma unroll
       for (int e = 0; e < 16; e++) {
-        const uint32_t m = m0 + wm * 64 + i * 32 + 8 * (e / 4) + 4 * (lane >> 5) + (e % 4);
-        if (m < p.M && n < p.N) p.out[(size_t)m * p.N + n] = (_Float16)tot[i][j][e];
+        // tile rows come in the groups of eight the activations were fetched in; a group moved
+        // back writes the values the group before it writes, to the same places
+        const uint32_t row0 = m0 + wm * 64 + i * 32 + 8 * (e / 4), last = p.M >= 8 ? p.M - 8 : 0;
+        const uint32_t m = (row0 < last ? row0 : last) + 4 * (lane >> 5) + (e % 4);
+        if (row0 < p.M && m < p.M && n < p.N) p.out[(size_t)m * p.N + n] = (_Float16)tot[i][j][e];
       }
     }
 }
@@ -450,7 +520,7 @@ hipError_t launch_tile(GemmParams p, bool affine, hipStream_t s) {
   p.mtiles = (p.M + TM - 1) / TM;
   p.ntiles = (p.N + TN - 1) / TN;
   const dim3 grid(p.mtiles * p.ntiles);
-  const size_t smem = NSTAGE * ((size_t)(TM + TN) * CHUNKS * 16 + (size_t)TN * (affine ? 1 : 2) * sizeof(float));
+  const size_t smem = NSTAGE * (size_t)(TM + TN) * CHUNKS * 16 + 2 * (size_t)TN * SCB * (affine ? 1 : 2) * sizeof(_Float16);  // stages + scale ring
   if (affine) {
     auto k = gemm_kernel<WM, WN, true>;
     if (smem > 64 * 1024) (void)hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
@@ -465,7 +535,10 @@ hipError_t launch_tile(GemmParams p, bool affine, hipStream_t s) {
 
 }  // namespace
 // 4-bit, f16 output, dense, K a multiple of 64.
-bool gemm_supports(const MatmulArgs& a) { return a.slots == 0 && a.bits == 4 && !a.out_f32 && a.K % KS == 0; }
+// The scales are fetched as 4-byte pairs, so a row of them must start on 4 bytes.
+bool gemm_supports(const MatmulArgs& a) {
+  return a.slots == 0 && a.bits == 4 && !a.out_f32 && a.K % KS == 0 && a.spr % 2 == 0;
+}
 
 static uint32_t xs_stride_of(const MatmulArgs& a) { return (2 * a.spr + KS - 1) / KS * KS; }
 
