@@ -121,6 +121,13 @@ __device__ __forceinline__ void static_for(F&& f) {
 }
 
 constexpr int NSTAGE = 3;
+// The value, made opaque to the compiler: what is computed from it inside the loop stays there
+// instead of being hoisted into a register that lives through the loop (the 256 x 128 tile runs
+// at the register limit, and a reload from scratch in the loop waits for every fetch in flight).
+__device__ __forceinline__ uint32_t opaque(uint32_t x) {
+  asm volatile("" : "+v"(x));
+  return x;
+}
 constexpr int SCB = 6;  // steps per batch of scales: two turns of the three LDS stages, so the hot loop has no branch
 
 // 16 bytes per lane from global memory (uniform base + 32-bit lane offset) straight into LDS slot
@@ -265,10 +272,10 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
   // of f16 (4 bytes) per lane and instruction, into batch slot (batch & 1) of the ring, laid out
   // [pair][column]. Pairs past a row's end repeat the row's last pair and are never used.
   const bool sc_loader = wave < TN / 64;
-  uint32_t sc_n = n0 + tid;
-  sc_n = sc_n < p.N ? sc_n : p.N - 1;
-  const uint32_t sc_off = sc_n * p.spr * 2u;  // spr is even (checked on the host): rows start on 4 bytes
   auto load_sc = [&](uint32_t batch) __attribute__((always_inline)) {
+    uint32_t sc_n = n0 + wave * 64 + opaque(lane);
+    sc_n = sc_n < p.N ? sc_n : p.N - 1;
+    const uint32_t sc_off = sc_n * p.spr * 2u;  // spr is even (checked on the host): rows start on 4 bytes
 #pragma unroll
     for (int k = 0; k < SC_PAIRS; k++) {
       uint32_t e = batch * (SCB * SCALES) + 2 * k;
@@ -286,7 +293,6 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
     a_rd[ks] = x + wm * 64 * ROW_BYTES;
     b_rd[ks] = x + W_BASE + wn * 64 * ROW_BYTES;
   }
-  const uint32_t sc_rd = SC_BASE + (wn * 64 + frow) * 4;
   auto read_a = [&](uint32_t stage, int i, int ks) __attribute__((always_inline)) {
     return *reinterpret_cast<const h8*>(smem + stage * STAGE_BYTES + a_rd[ks] + i * 32 * ROW_BYTES);
   };
@@ -406,7 +412,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
     if (fetch_sc && sc_loader) load_sc(batch + 1);
     {
       const uint32_t e = pos * SCALES;  // element of the batch: pair e / 2, half e % 2
-      const uint32_t at = sc_rd + (batch & 1u) * SC_BATCH + (e >> 1) * (TN * 4) + (e & 1u) * 2;
+      const uint32_t at = (opaque(lane) & 31u) * 4 + (SC_BASE + wn * 256 + (batch & 1u) * SC_BATCH + (e >> 1) * (TN * 4) + (e & 1u) * 2);
 #pragma unroll
       for (int j = 0; j < 2; j++) {
         scp[j] = sc[SCALES - 1][j];
