@@ -99,6 +99,10 @@ def test_auto_picks_a_family_by_rows(capi):
     assert capi.resolve(good(capi, M=300, bits=3, k_packed=384, scales_per_row=64)) == capi.KERNEL_SKINNY
     rc, why = capi.validate(good(capi, M=17, kernel=capi.KERNEL_ROWS))
     assert rc == capi.E_UNSUPPORTED and "rows" in why
+    # an odd number of scales per row (K = 192) is outside the tile GEMM: the default goes to the streaming kernel
+    odd = dict(M=300, k_packed=24, scales_per_row=3)
+    assert capi.resolve(good(capi, **odd)) == capi.KERNEL_SKINNY
+    assert capi.validate(good(capi, kernel=capi.KERNEL_GEMM, **odd))[0] == capi.E_UNSUPPORTED
 
 
 def test_no_device_is_a_loud_error(capi):

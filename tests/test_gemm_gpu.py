@@ -77,6 +77,36 @@ def test_gemm_one_hot_pins_staged_weights(ctx, capi, synth, oracle):
         assert np.array_equal(got, w16[:, ks].T)
 
 
+def test_odd_scale_count_leaves_the_tile_family(ctx, capi, synth, oracle):
+    """The tile GEMM fetches scales as 4-byte pairs, so rows of an odd number of scales (K = 192: three groups of
+    64) are not its to take: asked for by name it is refused, and the default routing serves them elsewhere."""
+    M, N, K = 140, 136, 192
+    A, w, s, b = make(synth, True, M, N, K)
+    desc = capi.MatmulDesc(bits=4, affine=1, kernel=capi.KERNEL_GEMM, M=M, N=N, k_packed=K // 8, scales_per_row=3,
+                           out=4096, in_=4096, scales=4096, weights=4096, biases=4096)
+    rc, why = capi.validate(desc)
+    assert rc == capi.E_UNSUPPORTED, why
+    desc.kernel = capi.KERNEL_AUTO
+    assert capi.resolve(desc) != capi.KERNEL_GEMM
+    got = run(ctx, capi, True, M, M, N, K, A, w, s, b, capi.KERNEL_AUTO)
+    ref = oracle.gemm(oracle.MODE_FORMULA_F64, 4, True, M, N, K, A, w, s, b, threads=8)
+    assert rel_err(got.view(np.float16).astype(np.float64), ref, 1e-2) < 1e-2
+
+
+@pytest.mark.parametrize("rows", [257, 264, 511])
+def test_rows_past_the_last_full_group(ctx, capi, synth, oracle, rows):
+    """256 x 128 tiles whose last tile holds 1, 8 or 255 rows: the fetch groups that reach past M are moved back
+    over valid rows and must neither disturb the rows they repeat nor write past M."""
+    N, K = 136, 256
+    A, w, s, b = make(synth, True, 512, N, K)
+    got = run(ctx, capi, True, rows, 512, N, K, A, w, s, b, capi.KERNEL_GEMM, prefill=0x5A)
+    ref = oracle.gemm(oracle.MODE_FORMULA_F64, 4, True, rows, N, K, A, w, s, b, threads=8)
+    assert rel_err(got[:rows].view(np.float16).astype(np.float64), ref, 1e-2) < 1e-2
+    assert (got[rows:] == 0x5A5A).all(), "rows past M were written"
+    full = run(ctx, capi, True, 512, 512, N, K, A, w, s, b, capi.KERNEL_GEMM)
+    assert np.array_equal(got[:rows], full[:rows]), "a row depends on how many rows follow it"
+
+
 @pytest.mark.parametrize("M", [128, 512])
 def test_config3_shape(ctx, capi, synth, oracle, M):
     """configs[2]: K=4096, N=14336; checked on a row sample against the formula and the f16-weight reference."""
