@@ -141,7 +141,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this path is built and measured on ONE GPU; --gpus %d is not supported "
-                         "(sharding is design-only, see DESIGN.md)" % args.gpus)
+                         "(a second GPU would own a column range of each weight matrix; nothing here uses one)" % args.gpus)
 
     pkg = importlib.import_module("zero-tvm_amd")
     capi = pkg.capi
