@@ -22,6 +22,25 @@ const put = (name) => { const b = load(name); const buf = dev.createBuffer(b.len
   if (!threw) throw new Error('affine pipeline without bias did not throw')
 }
 {
+  // boot-time GEMM probe on the dense weights: families timed with the family forced, pick stored and replayed
+  const { K, N } = meta.dense
+  const CAP = 256
+  const pipe = dev.createPipeline('int4_matmul_batched_dyn_affine')
+  const act = dev.createBuffer(CAP * K * 2, 'chunk'), out = dev.createBuffer(CAP * N * 2, 'chunk_out')
+  dev.fill(act, 0)
+  const group = dev.bg(pipe, [out, act, put('s.bin'), put('w.bin'), dev.uniformBuf(z.densePod(K, N, 4, true, CAP)), put('b.bin')])
+  const desc = dev.descriptor(group)
+  const timings = dev.probeFamilies(desc, ['gemm', 'skinny', 'rows', 'gemv'], [64, 256], { warmup: 1, rounds: 2 })
+  const store = z.fileTuneStore(path.join(dir, 'tune_store.json'))
+  const adapter = z.deviceFingerprint(dev.info())
+  let probes = 0
+  const runProbe = () => { probes++; return dev.probeFamilies(desc, ['gemm', 'skinny', 'gemv'], [64, 256], { warmup: 1, rounds: 2 }) }
+  const first = z.resolveTunedGemm({ specId: 'js-dense', runnable: ['gemm', 'skinny', 'gemv'], store, adapterId: adapter, runProbe })
+  const second = z.resolveTunedGemm({ specId: 'js-dense', runnable: ['gemm', 'skinny', 'gemv'], store, adapterId: adapter, runProbe })
+  fs.writeFileSync(path.join(dir, 'tune.json'), JSON.stringify({ timed: Object.keys(timings).sort(), first, second, probes, adapter,
+    sizes: Object.keys(timings.gemm || {}).map(Number) }))
+}
+{
   const { E, slots, tokens, d, ffn } = meta.moe
   const pipe = dev.createPipeline('int4_matmul_tiled_affine_moe')
   const out = dev.createBuffer(tokens * slots * 2 * ffn * 2, 'gu')

@@ -81,6 +81,12 @@ def test_js_dispatch_on_gpu(tmp_path, synth, oracle):
     y = np.fromfile(str(tmp_path / "y_dense.bin"), np.float16).astype(np.float64)
     ref = oracle.gemm(oracle.MODE_FORMULA_F32, 4, True, 1, N, K, x, w, s, b, threads=8)[0]
     assert rel_err(y, ref, 1e-2) < 1e-2
+    # the boot-time GEMM probe: the row-group family stops at 16 rows, the others are timed at both sizes; the pick is
+    # stored under the device's key and the second resolve replays it without probing again
+    tune = json.loads((tmp_path / "tune.json").read_text())
+    assert tune["timed"] == ["gemm", "gemv", "skinny"] and sorted(tune["sizes"]) == [64, 256]
+    assert tune["first"]["source"] == "probed" and tune["first"]["pick"] in ("gemm", "skinny")
+    assert tune["second"] == {"pick": tune["first"]["pick"], "source": "stored"} and tune["probes"] == 1 and tune["adapter"]
     ym = np.fromfile(str(tmp_path / "y_moe.bin"), np.float16).astype(np.float64).reshape(tokens, slots, 2, ffn)
     rm = oracle.moe_gemv(oracle.MODE_FORMULA_F32, 4, ffn, d, tokens, slots, (0, 2 * ffn, d, slots * 2 * ffn, slots), ids, mx,
                          mw, ms, mb, ym.size).reshape(tokens, slots, 2, ffn)

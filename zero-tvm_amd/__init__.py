@@ -6,6 +6,7 @@ The directory name carries a hyphen, so import it with
   host.capi    ctypes binding of the C ABI (lib/libztvm_hip.so)
   host.engine  mirror of the reference's dispatch surface (uniformBuf / bg / dispatch)
   host.synth   seeded synthetic tensors of the benchmark configurations
+  host.gemm_tune  boot-time choice of the prefill GEMM by measurement (policy of the reference's gemm-tune.ts)
   build        hipcc build recipe
 """
 from .host import capi  # noqa: F401

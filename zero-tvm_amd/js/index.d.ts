@@ -47,6 +47,9 @@ export declare class Device {
     headDim: number; ropeTheta: number }): void
   kvQuantizeInt8(bufs: BindEntry[], pod: Uniform, model: { kvHeads: number; headDim: number; pageSize: number },
     tokens?: number): void
+  matmul(desc: MatmulDesc): void
+  probeFamilies(desc: MatmulDesc, families: KernelFamily[], Ms?: number[],
+    opts?: { warmup?: number; rounds?: number }): TuneTimings
   beginEncoder(): void
   finishEncoder(): unknown
   submit(cmdbuf: unknown): void
@@ -66,6 +69,25 @@ export declare function resolveChunkCap(opts: { chunkCap?: number }, spec: { max
 export type ChunkGemmName = 'e5' | 'sgmat' | 'tiled' | 'matvec'
 export declare function pickChunkGemm(caps: { want?: ChunkGemmName; chunkTiled: boolean; dimsOK: boolean; capTiles64: boolean
   e5Ready: boolean; sgmatReady: boolean; cap: number }): { used: ChunkGemmName; rejected: string | null }
+export type KernelFamily = 'gemm' | 'skinny' | 'rows' | 'gemv'
+export type TuneTimings = { [candidate: string]: { [m: number]: number[] } }
+export interface TuneStore { load(key: string): string | null; save(key: string, value: string): void }
+export declare const TUNE_VERSION: number
+export declare const TUNE_TTL_MS: number
+export declare const TUNE_MS: number[]
+export declare function tuneKey(adapterId: string, specId: string): string
+export declare function deviceFingerprint(info: { name?: string; computeUnits?: number; hbmBytes?: bigint } | null): string | null
+export declare function median(xs: number[]): number
+export declare function pickFromTimings(medians: { [candidate: string]: number[] }, ladder: string[]): string
+export declare function loadTunedPick(store: TuneStore | null, key: string, runnable: string[], now?: number): string | null
+export declare function saveTunedPick(store: TuneStore | null, key: string, pick: string, ms: { [c: string]: number },
+  candidates: string[]): void
+export declare function memoryTuneStore(init?: { [key: string]: string }): TuneStore
+export declare function fileTuneStore(file: string): TuneStore
+export declare function timeClosures(sync: () => void, runs: { [candidate: string]: (m: number) => void }, Ms: number[],
+  opts?: { warmup?: number; rounds?: number; clock?: () => number }): TuneTimings
+export declare function resolveTunedGemm(opts: { specId: string; runnable: string[]; explicit?: string; store?: TuneStore | null
+  adapterId?: string | null; order?: string[]; runProbe: () => TuneTimings }): { pick: string; source: 'explicit' | 'stored' | 'probed' } | null
 export declare function foldGridX(total: number, maxX?: number): { x: number; z: number }
 export declare function densePod(K: number, N: number, bits?: number, affine?: boolean, M?: number): number[]
 export declare function moePods(dModel: number, ffn: number, slots: number, bits?: number): { gate: number[]; down: number[] }

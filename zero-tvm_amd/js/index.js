@@ -9,6 +9,7 @@
 // and turns a (pipeline, bind group, grid) triple into one ztvm_matmul descriptor. Plain ES2019 CommonJS
 // so it loads on any Node with N-API >= 6; TypeScript callers use index.d.ts.
 const path = require('path')
+const tune = require('./gemm_tune')
 
 let native = null
 function addon() {
@@ -320,6 +321,15 @@ class Device {
   finishEncoder() { return addon().recordEnd(this.ctx) }
   submit(cmdbuf) { addon().submit(this.ctx, cmdbuf) }
   sync() { addon().sync(this.ctx) }
+
+  // one ztvm_matmul from a ready descriptor (what dispatch() builds from a pipeline and a bind group)
+  matmul(desc) { addon().matmul(this.ctx, desc) }
+
+  // Time this library's kernel families on `desc` (gemm_tune.js: probeFamilies) with this device's queue.
+  probeFamilies(desc, families, Ms, opts) {
+    return tune.probeFamilies({ validate: (d) => addon().validate(d), matmul: (d) => this.matmul(d), sync: () => this.sync() },
+      desc, families, Ms, opts)
+  }
 }
 
 function densePod(K, N, bits, affine, M) {
@@ -339,5 +349,10 @@ function moePods(dModel, ffn, slots, bits) {
 module.exports = {
   KERNEL, Device, Uniform, int4MatmulEntry, checkOpts, INT4_MATMUL_VARIANTS, GEMM_ENTRIES, INT8_ENTRIES, ALL_ENTRIES, createPipeline,
   resolveMatmul, resolveChunkCap, pickChunkGemm, foldGridX, densePod, moePods,
+  // boot-time choice of the prefill GEMM by measurement (gemm_tune.js)
+  TUNE_VERSION: tune.TUNE_VERSION, TUNE_TTL_MS: tune.TUNE_TTL_MS, TUNE_MS: tune.TUNE_MS, tuneKey: tune.tuneKey,
+  deviceFingerprint: tune.deviceFingerprint, median: tune.median, pickFromTimings: tune.pickFromTimings,
+  loadTunedPick: tune.loadTunedPick, saveTunedPick: tune.saveTunedPick, memoryTuneStore: tune.memoryTuneStore,
+  fileTuneStore: tune.fileTuneStore, timeClosures: tune.timeClosures, resolveTunedGemm: tune.resolveTunedGemm,
   validate: (desc) => addon().validate(desc), resolve: (desc) => addon().resolve(desc), abiVersion: () => addon().abiVersion(),
 }
