@@ -77,6 +77,24 @@ def test_gemm_one_hot_pins_staged_weights(ctx, capi, synth, oracle):
         assert np.array_equal(got, w16[:, ks].T)
 
 
+def test_seeded_random_shapes(ctx, capi, synth, oracle):
+    """Thirty seeded shapes through the tile family: every tile height (M up to 600 crosses the 64-, 128- and 256-row
+    tiles and their partial last tiles), ragged N, K from two scale pairs up, both formats; rows past M stay untouched."""
+    rng = np.random.default_rng(20240611)
+    for case in range(30):
+        affine = bool(case % 2)
+        M = int(rng.choice([1, 7, 8, 9, 63, 65, 129, 255, 257, 300, 511, 600]) if case < 12 else rng.integers(1, 601))
+        N = int(rng.integers(1, 420))
+        K = 128 * int(rng.choice([1, 2, 3, 5, 8, 11, 16]))
+        CAP = M + int(rng.integers(0, 9))
+        A, w, s, b = make(synth, affine, CAP, N, K)
+        got = run(ctx, capi, affine, M, CAP, N, K, A, w, s, b, capi.KERNEL_GEMM, prefill=0x5A)
+        ref = oracle.gemm(oracle.MODE_FORMULA_F64, 4, affine, M, N, K, A, w, s, b, threads=8)
+        err = rel_err(got[:M].view(np.float16).astype(np.float64), ref, 1e-2)
+        assert err < 1e-2, (case, affine, M, N, K, err)
+        assert (got[M:] == 0x5A5A).all(), (case, "rows past M were written")
+
+
 def test_odd_scale_count_leaves_the_tile_family(ctx, capi, synth, oracle):
     """The tile GEMM fetches scales as 4-byte pairs, so rows of an odd number of scales (K = 192: three groups of
     64) are not its to take: asked for by name it is refused, and the default routing serves them elsewhere."""
