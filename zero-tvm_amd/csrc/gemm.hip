@@ -293,11 +293,16 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
     a_rd[ks] = x + wm * 64 * ROW_BYTES;
     b_rd[ks] = x + W_BASE + wn * 64 * ROW_BYTES;
   }
+  // With a stage known at compile time the stage and block offsets fold into the instruction; the steps outside
+  // the hot loop pass a runtime stage and add it to the same address registers (opaque, so that the compiler does
+  // not rebuild the addresses from parts it would have to carry through the hot loop).
   auto read_a = [&](uint32_t stage, int i, int ks) __attribute__((always_inline)) {
-    return *reinterpret_cast<const h8*>(smem + stage * STAGE_BYTES + a_rd[ks] + i * 32 * ROW_BYTES);
+    if (__builtin_constant_p(stage)) return *reinterpret_cast<const h8*>(smem + stage * STAGE_BYTES + a_rd[ks] + i * 32 * ROW_BYTES);
+    return *reinterpret_cast<const h8*>(smem + (opaque(a_rd[ks]) + stage * STAGE_BYTES) + i * 32 * ROW_BYTES);
   };
   auto read_b = [&](uint32_t stage, int j, int ks) __attribute__((always_inline)) {
-    return *reinterpret_cast<const h8*>(smem + stage * STAGE_BYTES + b_rd[ks] + j * 32 * ROW_BYTES);
+    if (__builtin_constant_p(stage)) return *reinterpret_cast<const h8*>(smem + stage * STAGE_BYTES + b_rd[ks] + j * 32 * ROW_BYTES);
+    return *reinterpret_cast<const h8*>(smem + (opaque(b_rd[ks]) + stage * STAGE_BYTES) + j * 32 * ROW_BYTES);
   };
 
   f16v tot[2][2];
@@ -503,18 +508,20 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
 #pragma unroll
     for (int e = 0; e < 16; e++) tot[1][j][e] = __builtin_fmaf(sc[SCALES - 1][j], part[1][j][e], tot[1][j][e]);
 
-  // D layout of a 32x32 block: lane -> column n = lane % 32, register e -> row 8*(e/4) + 4*(lane/32) + e%4
+  // D layout of a 32x32 block: lane -> column n = lane % 32, register e -> row 8*(e/4) + 4*(lane/32) + e%4.
+  // The lane's part of the store addresses is computed here, not carried through the loop.
+  const uint32_t ln = opaque(lane);
 #pragma unroll
   for (int i = 0; i < 2; i++)
 #pragma unroll
     for (int j = 0; j < 2; j++) {
-      const uint32_t n = n0 + wn * 64 + j * 32 + (lane & 31u);
+      const uint32_t n = n0 + wn * 64 + j * 32 + (ln & 31u);
 #pragma unroll
       for (int e = 0; e < 16; e++) {
         // tile rows come in the groups of eight the activations were fetched in; a group moved
         // back writes the values the group before it writes, to the same places
         const uint32_t row0 = m0 + wm * 64 + i * 32 + 8 * (e / 4), last = p.M >= 8 ? p.M - 8 : 0;
-        const uint32_t m = (row0 < last ? row0 : last) + 4 * (lane >> 5) + (e % 4);
+        const uint32_t m = (row0 < last ? row0 : last) + 4 * (ln >> 5) + (e % 4);
         if (row0 < p.M && m < p.M && n < p.N) p.out[(size_t)m * p.N + n] = (_Float16)tot[i][j][e];
       }
     }
