@@ -51,7 +51,6 @@ struct Tune {
   int gemv_path = 0;        // 0/1: the f16 dot2 kernel; 2: the int8 matrix-core kernel (opt-in)
   int i8_ksplit = 0;        // waves sharing one tile in the int8 GEMV (1, 2 or 4)
   int i8_wg_per_cu = 0;
-  int skinny_wg_per_cu = 0;
   int skinny_ksplit = 0;     // workgroups sharing the k range of one skinny tile (0: chosen from M, N, K)
   int rows_wg_per_cu = 0;    // the row-group GEMV: workgroups per CU and waves per workgroup (0: chosen from the LDS it stages)
   int rows_waves = 0;

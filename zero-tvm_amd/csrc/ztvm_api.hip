@@ -168,7 +168,6 @@ const Option kOptions[] = {
     {"gemv.path", &Tune::gemv_path},
     {"i8.ksplit", &Tune::i8_ksplit},
     {"i8.wg_per_cu", &Tune::i8_wg_per_cu},
-    {"skinny.wg_per_cu", &Tune::skinny_wg_per_cu},
     {"skinny.ksplit", &Tune::skinny_ksplit},
     {"rows.wg_per_cu", &Tune::rows_wg_per_cu},
     {"rows.waves", &Tune::rows_waves},
