@@ -136,7 +136,7 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the per-shape, GEMM, MoE and int3 extras")
     ap.add_argument("--pmc", action="store_true",
                     help="counter-collection mode for `rocprofv3 --pmc`: a few eager launches of a 256 MiB copy "
-                         "(calibration) and of each configs[1] GEMV, no timing")
+                         "(calibration), of each configs[1] GEMV and of the M=512 prefill GEMM, no timing")
     ap.add_argument("--option", action="append", default=[], help="name=value launch knob (ztvm_set_option)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -164,6 +164,12 @@ def main():
             descs = [make_desc(capi, 4, K, N, 1, upload_set(ctx, synth, K, N, 4, salt=r)[0]) for r in range(4)]
             for r in range(8):
                 ctx.matmul(descs[r % 4])
+        # the prefill GEMM of configs[2] at M=512, for its own counters
+        K, N, M = 4096, 14336, 512
+        gdescs = [make_desc(capi, 4, K, N, M, upload_set(ctx, synth, K, N, 4, salt=r, M=M)[0], kernel=capi.KERNEL_GEMM)
+                  for r in range(2)]
+        for r in range(6):
+            ctx.matmul(gdescs[r % 2])
         ctx.sync()
         ctx.close()
         print(json.dumps({"pmc_mode": True, "copy_bytes": nbytes}))
