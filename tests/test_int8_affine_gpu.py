@@ -53,6 +53,41 @@ def test_batched_ragged_and_m_invariant(ctx, capi, synth, oracle):
     assert np.array_equal(outs[0][:M], outs[1][:M]), "M-variance"
 
 
+@pytest.mark.parametrize("M,CAP,N,K", [(6, 8, 64, 2560), (47, 64, 200, 1024), (130, 256, 136, 512), (300, 320, 264, 1024),
+                                       (257, 260, 136, 256), (511, 512, 392, 640)])
+def test_tile_gemm_family(ctx, capi, synth, oracle, M, CAP, N, K):
+    """The 8-bit form of the tile GEMM (bytes staged as exact f16 integers, two words per 16-byte chunk) against the
+    formula, at every tile height, with partial last tiles, ragged N, and rows past M untouched; a row does not
+    depend on how many rows follow it."""
+    x, w, s, b = make8(synth, N, K, CAP)
+    with Dev(ctx) as d:
+        X, W, S, B = d.put(x), d.put(w), d.put(s), d.put(b)
+        outs = []
+        for m in (M, CAP):
+            out = d.empty(CAP * N * 2, fill=0x5A)
+            ctx.matmul(desc8(capi, m, N, K, out, X, W, S, B, kernel=capi.KERNEL_GEMM))
+            outs.append(ctx.download(out, CAP * N * 2, np.uint16).reshape(CAP, N))
+    ref = oracle.gemm(oracle.MODE_FORMULA_F64, 8, True, M, N, K, x, w, s, b, threads=8)
+    assert rel_err(outs[0][:M].view(np.float16).astype(np.float64), ref, 1e-2) < 1e-2
+    assert (outs[0][M:] == 0x5A5A).all(), "rows past M were written"
+    assert np.array_equal(outs[0][:M], outs[1][:M]), "M-variance"
+
+
+def test_tile_gemm_one_hot_is_the_dequantized_weight(ctx, capi, synth, oracle):
+    """A = rows of the identity through the 8-bit tile GEMM: Y[m, n] = f16(fl32(q*s + b)) of W[n, k_m], bit for bit."""
+    N, K = 160, 256
+    _, w, s, b = make8(synth, N, K, 1)
+    ks = np.array([0, 1, 2, 3, 4, 7, 8, 15, 31, 32, 33, 63, 64, 65, 127, 128, 191, 200, 254, 255] * 4, np.int64)[:64]
+    A = np.zeros((64, K), np.float16)
+    A[np.arange(64), ks] = 1.0
+    with Dev(ctx) as d:
+        out = d.empty(64 * N * 2, fill=0)
+        ctx.matmul(desc8(capi, 64, N, K, out, d.put(A), d.put(w), d.put(s), d.put(b), kernel=capi.KERNEL_GEMM))
+        got = ctx.download(out, 64 * N * 2, np.uint16).reshape(64, N)
+    w16 = oracle.dequant_matrix(8, True, N, K, w, s, b, want="f16")
+    assert np.array_equal(got, w16[:, ks].T)
+
+
 def test_dequant_and_one_hot_are_bit_exact(ctx, capi, synth, oracle):
     N, K = 96, 256
     _, w, s, b = make8(synth, N, K, 1, regime="B")
@@ -99,10 +134,15 @@ def test_rules_and_routing(capi):
     ok = capi.MatmulDesc(bits=8, affine=1, M=1, N=64, k_packed=256, scales_per_row=16, out=4096, in_=4096, scales=4096,
                          weights=4096, biases=4096)
     assert capi.validate(ok)[0] == 0 and capi.resolve(ok) == capi.KERNEL_GEMV
+    ok.M = 100
+    assert capi.resolve(ok) == capi.KERNEL_SKINNY        # the weight-streaming kernel up to 128 rows
     ok.M = 300
-    assert capi.resolve(ok) == capi.KERNEL_SKINNY        # the weight-streaming kernel at any M; no 8-bit tile GEMM
+    assert capi.resolve(ok) == capi.KERNEL_GEMM          # the tile GEMM above
     ok.kernel = capi.KERNEL_GEMM
-    assert capi.validate(ok)[0] == capi.E_UNSUPPORTED
+    assert capi.validate(ok)[0] == 0
+    ok.out_f32 = 1
+    assert capi.validate(ok)[0] == capi.E_UNSUPPORTED    # f32 output is the streaming kernel's
+    ok.out_f32, ok.kernel = 0, capi.KERNEL_AUTO
     sym = capi.MatmulDesc(bits=8, affine=0, M=1, N=64, k_packed=256, scales_per_row=32, out=4096, in_=4096, scales=4096, weights=4096)
     rc, why = capi.validate(sym)
     assert rc == capi.E_INVALID and "8-bit requires affine" in why

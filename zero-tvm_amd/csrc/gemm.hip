@@ -20,6 +20,9 @@
 // xs[m,g] = sum_{k in g} x[m,k] is produced once by a pre-pass as an f16
 // (hi, lo) pair and multiplied by the f16 biases on the matrix cores too.
 //
+// 8-bit affine rows (the reference's int8_affine_batched pipeline, compiler.ts:429-430) run through
+// the same kernel: only the staging of the weight tile differs (two packed words per 16-byte chunk).
+//
 // Tiling
 //   workgroup  WM x WN waves, each wave a 64 x 64 output tile (2 x 2 blocks of
 //              v_mfma_f32_32x32x16_f16); A operand = activations, B operand =
@@ -80,6 +83,22 @@ __device__ __forceinline__ h8 unpack_word_natural(uint32_t w, uint32_t c_mixed) 
   const h2 p2 = as_h2(and_or(t23, 0x00F0000Fu, c_mixed)) - off;       // v4, v5
   const h2 p3 = as_h2(and_or(t23 >> 8, 0x00F0000Fu, c_mixed)) - off;  // v6, v7
   return (h8){p0.x, p0.y, p1.x, p1.y, p2.x, p2.y, p3.x, p3.y};
+}
+
+// Two words of four bytes each -> eight exact f16 integers in natural k order: 0x6400 | byte is 1024 + byte, the
+// low halves of the two masked views are (v0, v1), the high halves (v2, v3).
+__device__ __forceinline__ h8 unpack_bytes_natural(uint32_t w0, uint32_t w1, uint32_t c_1024) {
+  const h2 off = {(_Float16)1024.f, (_Float16)1024.f};
+  h2 q[4];
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    const uint32_t w = i ? w1 : w0;
+    const uint32_t even = and_or(w, 0x00FF00FFu, c_1024);       // v0 | v2
+    const uint32_t odd = and_or(w >> 8, 0x00FF00FFu, c_1024);   // v1 | v3
+    q[2 * i + 0] = as_h2(__builtin_amdgcn_perm(odd, even, 0x05040100u)) - off;  // v0, v1
+    q[2 * i + 1] = as_h2(__builtin_amdgcn_perm(odd, even, 0x07060302u)) - off;  // v2, v3
+  }
+  return (h8){q[0].x, q[0].y, q[1].x, q[1].y, q[2].x, q[2].y, q[3].x, q[3].y};
 }
 
 // Group sums of the activations, one row of xs_stride f16 per activation row:
@@ -149,17 +168,17 @@ __device__ __forceinline__ void dma4(const void* base_uniform, uint32_t off, uin
 // the first MFMA of the pair, 1 after the second). The thread's packed words are unpacked in the
 // first eight half-slots, evenly spaced; the 32 fold FMAs of a run are spread over the run's
 // half-slots that have no unpack (over all of them when every one has).
-template <int W_WORDS>
-constexpr bool has_unpack(int hs) { return hs < 8 && hs % (8 / W_WORDS) == 0; }
-template <int W_WORDS, int RUNH>
+template <int W_CH>
+constexpr bool has_unpack(int hs) { return hs < 8 && hs % (8 / W_CH) == 0; }
+template <int W_CH, int RUNH>
 constexpr int fold_upto(int hs) {  // FMAs of the run done before half-slot hs
   const int r0 = hs / RUNH * RUNH;
   int total = 0;
-  for (int k = r0; k < r0 + RUNH; k++) total += has_unpack<W_WORDS>(k) ? 0 : 1;
+  for (int k = r0; k < r0 + RUNH; k++) total += has_unpack<W_CH>(k) ? 0 : 1;
   const bool flat = total == 0;
   if (flat) total = RUNH;
   int before = 0;
-  for (int k = r0; k < hs; k++) before += flat ? 1 : (has_unpack<W_WORDS>(k) ? 0 : 1);
+  for (int k = r0; k < hs; k++) before += flat ? 1 : (has_unpack<W_CH>(k) ? 0 : 1);
   return 32 * before / total;
 }
 
@@ -174,15 +193,18 @@ struct Seq {
   static constexpr int GRP(int p) { return AFFINE ? 0 : p / 4; }
 };
 
-template <int WM, int WN, bool AFFINE>
+template <int WM, int WN, bool AFFINE, int BITS>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) {
+  static_assert(BITS == 4 || (BITS == 8 && AFFINE), "4-bit affine or symmetric, 8-bit affine");
   using S = Seq<AFFINE>;
   constexpr int WAVES = WM * WN, THREADS = 64 * WAVES;
   constexpr int TM = 64 * WM, TN = 64 * WN;
   constexpr int A_LOADS = TM * CHUNKS / THREADS;  // 16-byte direct-to-LDS loads per lane per step
-  constexpr int W_WORDS = TN * 8 / THREADS;       // packed words per thread per step
-  static_assert(A_LOADS >= 1 && (W_WORDS == 2 || W_WORDS == 4 || W_WORDS == 8), "tile/thread mismatch");
-  constexpr int W_TPR = 8 / W_WORDS;              // threads per weight row
+  constexpr int W_CH = TN * 8 / THREADS;          // 8-k chunks (16 bytes of f16 in LDS) per thread per step
+  constexpr int WPC = BITS / 4;                   // packed words per chunk
+  constexpr int W_WORDS = W_CH * WPC;             // packed words per thread per step
+  static_assert(A_LOADS >= 1 && (W_CH == 2 || W_CH == 4 || W_CH == 8), "tile/thread mismatch");
+  constexpr int W_TPR = 8 / W_CH;                 // threads per weight row
   constexpr int SCALES = AFFINE ? 1 : 2;          // groups per step
   constexpr uint32_t ROW_BYTES = CHUNKS * 16;
   constexpr uint32_t STAGE_BYTES = (TM + TN) * ROW_BYTES;
@@ -207,8 +229,9 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
   const uint32_t mt = id % p.mtiles, nt = id / p.mtiles;
   const uint32_t m0 = mt * TM, n0 = nt * TN;
 
-  uint32_t c_mixed;  // OR constant: 64 in the high half, 1024 in the low half
-  asm volatile("v_mov_b32 %0, 0x54006400" : "=v"(c_mixed));
+  uint32_t c_mixed;  // OR constant: 4-bit: 64 in the high half, 1024 in the low half; 8-bit: 1024 in both
+  if (BITS == 4) asm volatile("v_mov_b32 %0, 0x54006400" : "=v"(c_mixed));
+  else asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(c_mixed));
 
   // ---- activations: global -> LDS without passing registers. One instruction fills 64
   // consecutive 16-byte LDS slots (8 rows), slot = lane; the lane fetches the chunk that the
@@ -242,9 +265,9 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
   const __amdgpu_buffer_rsrc_t wres = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(p.weights), 0, p.N * p.k_packed * 4u, 0x00020000);
   const uint32_t w_off = (w_n * p.k_packed + w_part * W_WORDS) * 4u;
   uint32_t w_adv = 0;  // uniform, bytes
-  uint32_t w_dst[W_WORDS];
+  uint32_t w_dst[W_CH];
 #pragma unroll
-  for (int j = 0; j < W_WORDS; j++) w_dst[j] = W_BASE + w_row * ROW_BYTES + (((w_part * W_WORDS + j) ^ swz(w_row)) << 4);
+  for (int j = 0; j < W_CH; j++) w_dst[j] = W_BASE + w_row * ROW_BYTES + (((w_part * W_CH + j) ^ swz(w_row)) << 4);
 
   struct WRegs {
     uint32_t w[W_WORDS];
@@ -260,12 +283,16 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
         r.w[4 * q4 + 0] = v.x; r.w[4 * q4 + 1] = v.y; r.w[4 * q4 + 2] = v.z; r.w[4 * q4 + 3] = v.w;
       }
     }
-    w_adv += KS / 2;
+    w_adv += KS * BITS / 8;
   };
   auto store_w_words = [&](const WRegs& r, uint32_t stage, int j0, int j1) __attribute__((always_inline)) {
 #pragma unroll
-    for (int j = j0; j < j1; j++)
-      *reinterpret_cast<h8*>(smem + stage * STAGE_BYTES + w_dst[j]) = unpack_word_natural<AFFINE>(r.w[j], c_mixed);
+    for (int j = j0; j < j1; j++) {  // chunk j of the thread: one 4-bit word or two 8-bit words
+      h8 v;
+      if constexpr (BITS == 4) v = unpack_word_natural<AFFINE>(r.w[j], c_mixed);
+      else v = unpack_bytes_natural(r.w[2 * j], r.w[2 * j + 1], c_mixed);
+      *reinterpret_cast<h8*>(smem + stage * STAGE_BYTES + w_dst[j]) = v;
+    }
   };
 
   // ---- scales: the first TN / 64 waves fetch SCB steps of their 64 columns at a time, one pair
@@ -323,8 +350,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
 #pragma unroll
       for (int i = 0; i < A_LOADS; i++) dma16(p.xs16 + (size_t)a_row0[i] * p.xs_stride + bs * KS, xs_lane, lds_slot(0, i));
 #pragma unroll
-      for (int j = 0; j < W_WORDS; j++) {
-        const uint32_t col = bs * KS + (w_part * W_WORDS + j) * 8;  // column c meets b[n][c mod G]; zero past 2G
+      for (int j = 0; j < W_CH; j++) {
+        const uint32_t col = bs * KS + (w_part * W_CH + j) * 8;  // column c meets b[n][c mod G]; zero past 2G
         h8 v = {0, 0, 0, 0, 0, 0, 0, 0};
         if (col < 2 * G) {
           if (G % 8 == 0) {
@@ -378,11 +405,11 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
   };
   load_a(0);
   load_w(wcur);
-  store_w_words(wcur, 0, 0, W_WORDS);
+  store_w_words(wcur, 0, 0, W_CH);
   if (nsteps > 1) {
     load_a(1);
     load_w(wcur);
-    store_w_words(wcur, 1, 0, W_WORDS);
+    store_w_words(wcur, 1, 0, W_CH);
   }
   if (nsteps > 2) load_w(wcur);
   __builtin_amdgcn_s_waitcnt(0x0070);
@@ -435,7 +462,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
       constexpr bool from_last_step = pp < S::RUN;
       auto fold = [&](auto hs_c) __attribute__((always_inline)) {
         constexpr int hs = decltype(hs_c)::value;
-        constexpr int q0 = fold_upto<W_WORDS, RUNH>(hs), q1 = (hs + 1) % RUNH == 0 ? 32 : fold_upto<W_WORDS, RUNH>(hs + 1);
+        constexpr int q0 = fold_upto<W_CH, RUNH>(hs), q1 = (hs + 1) % RUNH == 0 ? 32 : fold_upto<W_CH, RUNH>(hs + 1);
 #pragma unroll
         for (int q = q0; q < q1; q++) {
           const int j = q / 16, e = q % 16;
@@ -445,8 +472,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
       };
       auto unpack = [&](auto hs_c) __attribute__((always_inline)) {
         constexpr int hs = decltype(hs_c)::value;
-        if constexpr (has_unpack<W_WORDS>(hs)) {
-          constexpr int j = hs / (8 / W_WORDS);
+        if constexpr (has_unpack<W_CH>(hs)) {
+          constexpr int j = hs / (8 / W_CH);
           if (HOT || fetch_a) store_w_words(wcur, fill, j, j + 1);
         }
       };
@@ -527,30 +554,32 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
     }
 }
 
-template <int WM, int WN>
-hipError_t launch_tile(GemmParams p, bool affine, hipStream_t s) {
+template <int WM, int WN, bool AFFINE, int BITS>
+hipError_t launch_kernel(const GemmParams& p, hipStream_t s) {
   constexpr int TM = 64 * WM, TN = 64 * WN, THREADS = 64 * WM * WN;
-  p.mtiles = (p.M + TM - 1) / TM;
-  p.ntiles = (p.N + TN - 1) / TN;
-  const dim3 grid(p.mtiles * p.ntiles);
-  const size_t smem = NSTAGE * (size_t)(TM + TN) * CHUNKS * 16 + 2 * (size_t)TN * SCB * (affine ? 1 : 2) * sizeof(_Float16);  // stages + scale ring
-  if (affine) {
-    auto k = gemm_kernel<WM, WN, true>;
-    if (smem > 64 * 1024) (void)hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    hipLaunchKernelGGL(k, grid, dim3(THREADS), smem, s, p);
-  } else {
-    auto k = gemm_kernel<WM, WN, false>;
-    if (smem > 64 * 1024) (void)hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    hipLaunchKernelGGL(k, grid, dim3(THREADS), smem, s, p);
-  }
+  // stages + scale ring
+  const size_t smem = NSTAGE * (size_t)(TM + TN) * CHUNKS * 16 + 2 * (size_t)TN * SCB * (AFFINE ? 1 : 2) * sizeof(_Float16);
+  auto k = gemm_kernel<WM, WN, AFFINE, BITS>;
+  if (smem > 64 * 1024) (void)hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+  hipLaunchKernelGGL(k, dim3(p.mtiles * p.ntiles), dim3(THREADS), smem, s, p);
   return hipGetLastError();
 }
 
+template <int WM, int WN>
+hipError_t launch_tile(GemmParams p, bool affine, uint32_t bits, hipStream_t s) {
+  constexpr int TM = 64 * WM, TN = 64 * WN;
+  p.mtiles = (p.M + TM - 1) / TM;
+  p.ntiles = (p.N + TN - 1) / TN;
+  if (bits == 8) return launch_kernel<WM, WN, true, 8>(p, s);
+  if (affine) return launch_kernel<WM, WN, true, 4>(p, s);
+  return launch_kernel<WM, WN, false, 4>(p, s);
+}
+
 }  // namespace
-// 4-bit, f16 output, dense, K a multiple of 64.
+// 4-bit (affine or symmetric) or 8-bit affine, f16 output, dense, K a multiple of 64.
 // The scales are fetched as 4-byte pairs, so a row of them must start on 4 bytes.
 bool gemm_supports(const MatmulArgs& a) {
-  return a.slots == 0 && a.bits == 4 && !a.out_f32 && a.K % KS == 0 && a.spr % 2 == 0;
+  return a.slots == 0 && (a.bits == 4 || (a.bits == 8 && a.affine)) && !a.out_f32 && a.K % KS == 0 && a.spr % 2 == 0;
 }
 
 static uint32_t xs_stride_of(const MatmulArgs& a) { return (2 * a.spr + KS - 1) / KS * KS; }
@@ -576,10 +605,10 @@ hipError_t launch_gemm(const MatmulArgs& a, const Tune& t, void* scratch, hipStr
   int tile = t.gemm_tile;
   if (!tile) tile = a.M > 256 ? 3 : (a.M > 64 ? 2 : 1);  // measured: 256x128 wins from M=512 up
   switch (tile) {
-    case 3: return launch_tile<4, 2>(p, a.affine, s);  // 256 x 128, 8 waves
-    case 2: return launch_tile<2, 2>(p, a.affine, s);  // 128 x 128, 4 waves
-    case 4: return launch_tile<2, 4>(p, a.affine, s);  // 128 x 256, 8 waves
-    default: return launch_tile<1, 2>(p, a.affine, s);  // 64 x 128, 2 waves
+    case 3: return launch_tile<4, 2>(p, a.affine, a.bits, s);  // 256 x 128, 8 waves
+    case 2: return launch_tile<2, 2>(p, a.affine, a.bits, s);  // 128 x 128, 4 waves
+    case 4: return launch_tile<2, 4>(p, a.affine, a.bits, s);  // 128 x 256, 8 waves
+    default: return launch_tile<1, 2>(p, a.affine, a.bits, s);  // 64 x 128, 2 waves
   }
 }
 
