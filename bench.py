@@ -338,8 +338,8 @@ def main():
                                            "hbm_frac": round(gbytes / ms_g / 1e6 / HBM_PEAK_GBS, 4),
                                            "with_add_rmsnorm_prologue_us": round(ms_p * 1e3, 2)}
         # small batches: the row-group GEMV (M <= 16) and the weight-streaming matrix-core kernel (M <= 128); int4,
-        # configs[4]'s int3 M=8, and 8-bit rows (M=512: the 8-bit form of the tile GEMM)
-        for bits, M in ((4, 2), (4, 4), (4, 8), (4, 16), (4, 32), (4, 128), (3, 8), (8, 8), (8, 128), (8, 512)):
+        # configs[4]'s int3 M=8, and 8-bit rows (M=512: the 3-bit and 8-bit forms of the tile GEMM)
+        for bits, M in ((4, 2), (4, 4), (4, 8), (4, 16), (4, 32), (4, 128), (3, 8), (3, 512), (8, 8), (8, 128), (8, 512)):
             if bits == 4:
                 descs = [make_desc(capi, 4, 4096, 14336, M, b) for b, _ in gsets]
                 host0 = gsets[0][1]

@@ -95,6 +95,48 @@ def test_seeded_random_shapes(ctx, capi, synth, oracle):
         assert (got[M:] == 0x5A5A).all(), (case, "rows past M were written")
 
 
+def run3(ctx, capi, M, CAP, N, K, A, w, s, b, kernel, prefill=0):
+    with Dev(ctx) as d:
+        out = d.empty(CAP * N * 2, fill=prefill)
+        desc = capi.MatmulDesc(bits=3, affine=1, kernel=kernel, M=M, N=N, k_packed=3 * K // 32, scales_per_row=K // 64, out=out,
+                               in_=d.put(A), scales=d.put(s), weights=d.put(w), biases=d.put(b))
+        ctx.matmul(desc)
+        return ctx.download(out, CAP * N * 2, np.uint16).reshape(CAP, N)
+
+
+@pytest.mark.parametrize("M,CAP,N,K", [(6, 8, 64, 2560), (47, 64, 200, 1024), (130, 256, 136, 512), (300, 320, 264, 1024),
+                                       (257, 260, 136, 256), (511, 512, 392, 640)])
+def test_three_bit_tile_gemm(ctx, capi, synth, oracle, M, CAP, N, K):
+    """The 3-bit form (24-bit windows of the row bitstream, fetched as the dwords that cover a thread's bytes) against
+    the formula at every tile height, with rows past M untouched and no dependence on the rows that follow."""
+    A = synth.activations(CAP, K)
+    w = synth.packed_weights(N, K, bits=3)
+    s = synth.scales(N, K)
+    b = synth.biases(N, K, s, "A")
+    got = run3(ctx, capi, M, CAP, N, K, A, w, s, b, capi.KERNEL_GEMM, prefill=0x5A)
+    full = run3(ctx, capi, CAP, CAP, N, K, A, w, s, b, capi.KERNEL_GEMM)
+    ref = oracle.gemm(oracle.MODE_FORMULA_F64, 3, True, M, N, K, A, w, s, b, threads=8)
+    assert rel_err(got[:M].view(np.float16).astype(np.float64), ref, 1e-2) < 1e-2
+    assert (got[M:] == 0x5A5A).all(), "rows past M were written"
+    assert np.array_equal(got[:M], full[:M]), "M-variance"
+
+
+def test_three_bit_one_hot_is_the_dequantized_weight(ctx, capi, synth, oracle):
+    """Rows of the identity through the 3-bit tile GEMM return f16(fl32(q*s + b)) bit for bit, at k positions on
+    both sides of every word boundary of the bitstream."""
+    N, K = 160, 256
+    w = synth.packed_weights(N, K, bits=3)
+    s = synth.scales(N, K)
+    b = synth.biases(N, K, s, "A")
+    ks = np.array([0, 1, 7, 8, 9, 10, 11, 15, 20, 21, 22, 31, 32, 33, 42, 43, 63, 64, 65, 85, 86, 127, 128, 191, 200, 255] * 3,
+                  np.int64)[:64]
+    A = np.zeros((64, K), np.float16)
+    A[np.arange(64), ks] = 1.0
+    got = run3(ctx, capi, 64, 64, N, K, A.view(np.uint16), w, s, b, capi.KERNEL_GEMM)
+    w16 = oracle.dequant_matrix(3, True, N, K, w, s, b, want="f16")
+    assert np.array_equal(got, w16[:, ks].T)
+
+
 def test_odd_scale_count_leaves_the_tile_family(ctx, capi, synth, oracle):
     """The tile GEMM fetches scales as 4-byte pairs, so rows of an odd number of scales (K = 192: three groups of
     64) are not its to take: asked for by name it is refused, and the default routing serves them elsewhere."""

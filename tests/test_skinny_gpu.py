@@ -119,7 +119,7 @@ def test_auto_picks_skinny(capi):
         assert capi.resolve(desc) == want, M
     desc = capi.MatmulDesc(bits=3, affine=1, M=300, N=256, k_packed=48, scales_per_row=8, out=4096, in_=4096, scales=4096,
                            weights=4096, biases=4096)
-    assert capi.resolve(desc) == capi.KERNEL_SKINNY  # the tile GEMM has no 3-bit path
+    assert capi.resolve(desc) == capi.KERNEL_GEMM  # 3-bit rows: the same ladder
     for M, want in ((20, capi.KERNEL_SKINNY), (300, capi.KERNEL_GEMM)):  # 8-bit rows: the same ladder as 4-bit
         desc = capi.MatmulDesc(bits=8, affine=1, M=M, N=256, k_packed=128, scales_per_row=8, out=4096, in_=4096, scales=4096,
                                weights=4096, biases=4096)

@@ -20,8 +20,9 @@
 // xs[m,g] = sum_{k in g} x[m,k] is produced once by a pre-pass as an f16
 // (hi, lo) pair and multiplied by the f16 biases on the matrix cores too.
 //
-// 8-bit affine rows (the reference's int8_affine_batched pipeline, compiler.ts:429-430) run through
-// the same kernel: only the staging of the weight tile differs (two packed words per 16-byte chunk).
+// 8-bit affine rows (the reference's int8_affine_batched pipeline, compiler.ts:429-430) and 3-bit
+// affine rows (the q3 bitstream, int4_matmul.gen.ts:409-448) run through the same kernel: only the
+// staging of the weight tile differs (two packed words, or a 24-bit window, per 16-byte chunk).
 //
 // Tiling
 //   workgroup  WM x WN waves, each wave a 64 x 64 output tile (2 x 2 blocks of
@@ -99,6 +100,14 @@ __device__ __forceinline__ h8 unpack_bytes_natural(uint32_t w0, uint32_t w1, uin
     q[2 * i + 1] = as_h2(__builtin_amdgcn_perm(odd, even, 0x07060302u)) - off;  // v2, v3
   }
   return (h8){q[0].x, q[0].y, q[1].x, q[1].y, q[2].x, q[2].y, q[3].x, q[3].y};
+}
+
+// A window of eight 3-bit values (value i at bits [3i, 3i+3); bits from 24 up may hold anything) -> eight exact f16
+// integers in natural k order: the shared unpack returns the pairs (v0,v4) (v1,v5) (v2,v6) (v3,v7).
+__device__ __forceinline__ h8 unpack_q3_natural(uint32_t win, const UnpackConsts& uc) {
+  h2 q[4];
+  unpack3_views(win << 4, win >> 2, q, uc);
+  return (h8){q[0].x, q[1].x, q[2].x, q[3].x, q[0].y, q[1].y, q[2].y, q[3].y};
 }
 
 // Group sums of the activations, one row of xs_stride f16 per activation row:
@@ -195,14 +204,15 @@ struct Seq {
 
 template <int WM, int WN, bool AFFINE, int BITS>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) {
-  static_assert(BITS == 4 || (BITS == 8 && AFFINE), "4-bit affine or symmetric, 8-bit affine");
+  static_assert(BITS == 4 || ((BITS == 8 || BITS == 3) && AFFINE), "4-bit affine or symmetric, 8-bit and 3-bit affine");
   using S = Seq<AFFINE>;
   constexpr int WAVES = WM * WN, THREADS = 64 * WAVES;
   constexpr int TM = 64 * WM, TN = 64 * WN;
   constexpr int A_LOADS = TM * CHUNKS / THREADS;  // 16-byte direct-to-LDS loads per lane per step
   constexpr int W_CH = TN * 8 / THREADS;          // 8-k chunks (16 bytes of f16 in LDS) per thread per step
-  constexpr int WPC = BITS / 4;                   // packed words per chunk
-  constexpr int W_WORDS = W_CH * WPC;             // packed words per thread per step
+  // words fetched per thread and step: one (4-bit) or two (8-bit) per chunk; 3-bit chunks are 3 bytes of the row's
+  // bitstream, so a thread's 3 * W_CH bytes are fetched as the dwords that cover them
+  constexpr int W_WORDS = BITS == 3 ? (W_CH == 2 ? 2 : 3 * W_CH / 4) : W_CH * BITS / 4;
   static_assert(A_LOADS >= 1 && (W_CH == 2 || W_CH == 4 || W_CH == 8), "tile/thread mismatch");
   constexpr int W_TPR = 8 / W_CH;                 // threads per weight row
   constexpr int SCALES = AFFINE ? 1 : 2;          // groups per step
@@ -229,6 +239,11 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
   const uint32_t mt = id % p.mtiles, nt = id / p.mtiles;
   const uint32_t m0 = mt * TM, n0 = nt * TN;
 
+  UnpackConsts uc3;  // 3-bit: the two OR constants of the shared unpack
+  if (BITS == 3) {
+    asm volatile("v_mov_b32 %0, 0x64005400" : "=v"(uc3.c3_a));
+    asm volatile("v_mov_b32 %0, 0x58004800" : "=v"(uc3.c3_b));
+  }
   uint32_t c_mixed;  // OR constant: 4-bit: 64 in the high half, 1024 in the low half; 8-bit: 1024 in both
   if (BITS == 4) asm volatile("v_mov_b32 %0, 0x54006400" : "=v"(c_mixed));
   else asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(c_mixed));
@@ -263,7 +278,9 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
   w_n = w_n < p.N ? w_n : p.N - 1;  // clamped rows are never stored
   // one descriptor + 32-bit lane offset + uniform step offset: no address arithmetic in the loop
   const __amdgpu_buffer_rsrc_t wres = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(p.weights), 0, p.N * p.k_packed * 4u, 0x00020000);
-  const uint32_t w_off = (w_n * p.k_packed + w_part * W_WORDS) * 4u;
+  const uint32_t w_byte = w_n * p.k_packed * 4u + w_part * (W_CH * BITS);  // W_CH chunks of BITS bytes each
+  const uint32_t w_off = w_byte & ~3u;
+  const uint32_t w_sh = (w_byte & 3u) * 8;  // 3-bit with two chunks per thread: 0 or 16; otherwise 0
   uint32_t w_adv = 0;  // uniform, bytes
   uint32_t w_dst[W_CH];
 #pragma unroll
@@ -276,6 +293,12 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
     if (W_WORDS == 2) {
       const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(wres, w_off, w_adv, 0);
       r.w[0] = v.x; r.w[1] = v.y;
+    } else if (BITS == 3) {
+#pragma unroll
+      for (int q3 = 0; q3 < W_WORDS / 3; q3++) {
+        const u32x3 v = __builtin_amdgcn_raw_buffer_load_b96(wres, w_off + 12 * q3, w_adv, 0);
+        r.w[3 * q3 + 0] = v.x; r.w[3 * q3 + 1] = v.y; r.w[3 * q3 + 2] = v.z;
+      }
     } else {
 #pragma unroll
       for (int q4 = 0; q4 < W_WORDS / 4; q4++) {
@@ -283,14 +306,27 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
         r.w[4 * q4 + 0] = v.x; r.w[4 * q4 + 1] = v.y; r.w[4 * q4 + 2] = v.z; r.w[4 * q4 + 3] = v.w;
       }
     }
-    w_adv += KS * BITS / 8;
+    w_adv += KS * BITS / 8;  // bytes of a row per step
   };
   auto store_w_words = [&](const WRegs& r, uint32_t stage, int j0, int j1) __attribute__((always_inline)) {
 #pragma unroll
     for (int j = j0; j < j1; j++) {  // chunk j of the thread: one 4-bit word or two 8-bit words
       h8 v;
-      if constexpr (BITS == 4) v = unpack_word_natural<AFFINE>(r.w[j], c_mixed);
-      else v = unpack_bytes_natural(r.w[2 * j], r.w[2 * j + 1], c_mixed);
+      if constexpr (BITS == 4) {
+        v = unpack_word_natural<AFFINE>(r.w[j], c_mixed);
+      } else if constexpr (BITS == 8) {
+        v = unpack_bytes_natural(r.w[2 * j], r.w[2 * j + 1], c_mixed);
+      } else {
+        // chunk j of the thread is the 24-bit window at bit 24 * j of its bytes: four windows per three dwords
+        const int g = j / 4 * 3, jj = j % 4;
+        uint32_t d0 = r.w[g], d1 = r.w[g + 1], d2 = W_CH == 2 ? 0u : r.w[W_CH == 2 ? g : g + 2];
+        if (W_CH == 2) {  // the thread's six bytes start at bit 0 or 16 of its two dwords
+          d0 = __builtin_amdgcn_alignbit(d1, d0, w_sh);
+          d1 = d1 >> w_sh;
+        }
+        const uint32_t win = jj == 0 ? d0 : jj == 1 ? __builtin_amdgcn_alignbit(d1, d0, 24) : jj == 2 ? __builtin_amdgcn_alignbit(d2, d1, 16) : d2 >> 8;
+        v = unpack_q3_natural(win, uc3);
+      }
       *reinterpret_cast<h8*>(smem + stage * STAGE_BYTES + w_dst[j]) = v;
     }
   };
@@ -571,15 +607,16 @@ hipError_t launch_tile(GemmParams p, bool affine, uint32_t bits, hipStream_t s) 
   p.mtiles = (p.M + TM - 1) / TM;
   p.ntiles = (p.N + TN - 1) / TN;
   if (bits == 8) return launch_kernel<WM, WN, true, 8>(p, s);
+  if (bits == 3) return launch_kernel<WM, WN, true, 3>(p, s);
   if (affine) return launch_kernel<WM, WN, true, 4>(p, s);
   return launch_kernel<WM, WN, false, 4>(p, s);
 }
 
 }  // namespace
-// 4-bit (affine or symmetric) or 8-bit affine, f16 output, dense, K a multiple of 64.
+// 4-bit (affine or symmetric), 8-bit or 3-bit affine, f16 output, dense, K a multiple of 64.
 // The scales are fetched as 4-byte pairs, so a row of them must start on 4 bytes.
 bool gemm_supports(const MatmulArgs& a) {
-  return a.slots == 0 && (a.bits == 4 || (a.bits == 8 && a.affine)) && !a.out_f32 && a.K % KS == 0 && a.spr % 2 == 0;
+  return a.slots == 0 && (a.bits == 4 || ((a.bits == 8 || a.bits == 3) && a.affine)) && !a.out_f32 && a.K % KS == 0 && a.spr % 2 == 0;
 }
 
 static uint32_t xs_stride_of(const MatmulArgs& a) { return (2 * a.spr + KS - 1) / KS * KS; }
