@@ -64,6 +64,7 @@ struct GemmParams {
   uint32_t M, N, K, k_packed, spr;
   uint32_t mtiles, ntiles, nsteps, bias_steps, xs_stride;
   uint32_t xcd_swizzle;
+  uint32_t out_f32;  // the output is float instead of f16
 };
 
 // LDS swizzle: a 128-bit read serves 16 lanes per cycle = two 128-byte rows of banks, and rows of
@@ -585,7 +586,10 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
         // back writes the values the group before it writes, to the same places
         const uint32_t row0 = m0 + wm * 64 + i * 32 + 8 * (e / 4), last = p.M >= 8 ? p.M - 8 : 0;
         const uint32_t m = (row0 < last ? row0 : last) + 4 * (ln >> 5) + (e % 4);
-        if (row0 < p.M && m < p.M && n < p.N) p.out[(size_t)m * p.N + n] = (_Float16)tot[i][j][e];
+        if (row0 < p.M && m < p.M && n < p.N) {
+          if (p.out_f32) reinterpret_cast<float*>(p.out)[(size_t)m * p.N + n] = tot[i][j][e];
+          else p.out[(size_t)m * p.N + n] = (_Float16)tot[i][j][e];
+        }
       }
     }
 }
@@ -613,10 +617,10 @@ hipError_t launch_tile(GemmParams p, bool affine, uint32_t bits, hipStream_t s) 
 }
 
 }  // namespace
-// 4-bit (affine or symmetric), 8-bit or 3-bit affine, f16 output, dense, K a multiple of 64.
+// 4-bit (affine or symmetric), 8-bit or 3-bit affine, f16 or f32 output, dense, K a multiple of 64.
 // The scales are fetched as 4-byte pairs, so a row of them must start on 4 bytes.
 bool gemm_supports(const MatmulArgs& a) {
-  return a.slots == 0 && (a.bits == 4 || ((a.bits == 8 || a.bits == 3) && a.affine)) && !a.out_f32 && a.K % KS == 0 && a.spr % 2 == 0;
+  return a.slots == 0 && (a.bits == 4 || ((a.bits == 8 || a.bits == 3) && a.affine)) && a.K % KS == 0 && a.spr % 2 == 0;
 }
 
 static uint32_t xs_stride_of(const MatmulArgs& a) { return (2 * a.spr + KS - 1) / KS * KS; }
@@ -633,6 +637,7 @@ hipError_t launch_gemm(const MatmulArgs& a, const Tune& t, void* scratch, hipStr
   p.xs_stride = xs_stride_of(a);
   p.bias_steps = a.affine ? p.xs_stride / KS : 0;
   p.xcd_swizzle = t.gemm_xcd_swizzle;
+  p.out_f32 = a.out_f32 ? 1u : 0u;
   if (a.affine) {
     const uint32_t pad = p.xs_stride - 2 * a.spr, cpr = a.K / 8;
     const uint32_t n = a.M * (cpr > pad ? cpr : pad);  // one thread per chunk, and enough for the padding columns
