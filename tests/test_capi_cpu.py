@@ -97,7 +97,7 @@ def test_auto_picks_a_family_by_rows(capi):
         assert capi.resolve(good(capi, M=M)) == want, M
     assert capi.resolve(good(capi, M=8, bits=3, k_packed=384, scales_per_row=64)) == capi.KERNEL_ROWS
     assert capi.resolve(good(capi, M=300, bits=3, k_packed=384, scales_per_row=64)) == capi.KERNEL_GEMM
-    assert capi.resolve(good(capi, M=300, bits=3, k_packed=384, scales_per_row=64, out_f32=1)) == capi.KERNEL_GEMM
+    assert capi.resolve(good(capi, M=300, bits=3, k_packed=384, scales_per_row=64, out_f32=1)) == capi.KERNEL_SKINNY
     rc, why = capi.validate(good(capi, M=17, kernel=capi.KERNEL_ROWS))
     assert rc == capi.E_UNSUPPORTED and "rows" in why
     # an odd number of scales per row (K = 192) is outside the tile GEMM: the default goes to the streaming kernel

@@ -137,30 +137,6 @@ def test_three_bit_one_hot_is_the_dequantized_weight(ctx, capi, synth, oracle):
     assert np.array_equal(got, w16[:, ks].T)
 
 
-@pytest.mark.parametrize("bits,affine", [(4, True), (4, False), (3, True), (8, True)])
-def test_f32_output(ctx, capi, synth, oracle, bits, affine):
-    """The totals stored as f32: within f32 accumulation noise of the formula, and the f16 output is their rounding."""
-    M, N, K = 300, 264, 1024
-    A = synth.activations(M, K)
-    w = synth.packed_weights(N, K, bits=bits)
-    s = synth.scales(N, K, affine=affine, **(dict(lo=0.01, hi=0.06) if bits == 8 else {}))
-    b = synth.biases(N, K, s, "A") if affine else None
-    outs = []
-    with Dev(ctx) as d:
-        X, W, S, B = d.put(A), d.put(w), d.put(s), (d.put(b) if affine else 0)
-        for f32 in (0, 1):
-            out = d.empty((M + 1) * N * (4 if f32 else 2), fill=0x5A)
-            ctx.matmul(capi.MatmulDesc(bits=bits, affine=int(affine), out_f32=f32, kernel=capi.KERNEL_GEMM, M=M, N=N,
-                                       k_packed=K * bits // 32, scales_per_row=K // (64 if affine else 32), out=out, in_=X, scales=S,
-                                       weights=W, biases=B))
-            outs.append(ctx.download(out, (M + 1) * N * (4 if f32 else 2), np.uint32 if f32 else np.uint16).reshape(M + 1, N))
-    ref = oracle.gemm(oracle.MODE_FORMULA_F64, bits, affine, M, N, K, A, w, s, b, threads=8)
-    y32 = outs[1][:M].view(np.float32)
-    assert rel_err(y32.astype(np.float64), ref, 1.0) < (4e-5 if bits == 8 else 1e-5)
-    assert np.array_equal(y32.astype(np.float16).view(np.uint16), outs[0][:M]), "the f16 output is not the rounded f32 total"
-    assert (outs[1][M:] == 0x5A5A5A5A).all() and (outs[0][M:] == 0x5A5A).all(), "rows past M were written"
-
-
 def test_odd_scale_count_leaves_the_tile_family(ctx, capi, synth, oracle):
     """The tile GEMM fetches scales as 4-byte pairs, so rows of an odd number of scales (K = 192: three groups of
     64) are not its to take: asked for by name it is refused, and the default routing serves them elsewhere."""

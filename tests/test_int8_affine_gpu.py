@@ -141,7 +141,7 @@ def test_rules_and_routing(capi):
     ok.kernel = capi.KERNEL_GEMM
     assert capi.validate(ok)[0] == 0
     ok.out_f32 = 1
-    assert capi.validate(ok)[0] == 0                     # f32 output too
+    assert capi.validate(ok)[0] == capi.E_UNSUPPORTED    # f32 output is the streaming kernel's
     ok.out_f32, ok.kernel = 0, capi.KERNEL_AUTO
     sym = capi.MatmulDesc(bits=8, affine=0, M=1, N=64, k_packed=256, scales_per_row=32, out=4096, in_=4096, scales=4096, weights=4096)
     rc, why = capi.validate(sym)

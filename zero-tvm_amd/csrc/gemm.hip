@@ -64,7 +64,6 @@ struct GemmParams {
   uint32_t M, N, K, k_packed, spr;
   uint32_t mtiles, ntiles, nsteps, bias_steps, xs_stride;
   uint32_t xcd_swizzle;
-  uint32_t out_f32;  // the output is float instead of f16
 };
 
 // LDS swizzle: a 128-bit read serves 16 lanes per cycle = two 128-byte rows of banks, and rows of
@@ -281,7 +280,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
   const __amdgpu_buffer_rsrc_t wres = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(p.weights), 0, p.N * p.k_packed * 4u, 0x00020000);
   const uint32_t w_byte = w_n * p.k_packed * 4u + w_part * (W_CH * BITS);  // W_CH chunks of BITS bytes each
   const uint32_t w_off = w_byte & ~3u;
-  const uint32_t w_sh = (w_byte & 3u) * 8;  // 3-bit with two chunks per thread: 0 or 16; otherwise 0
+  // (w_byte & 3) is nonzero only for 3-bit rows with two chunks (six bytes) per thread: 2 for odd w_part
   uint32_t w_adv = 0;  // uniform, bytes
   uint32_t w_dst[W_CH];
 #pragma unroll
@@ -321,7 +320,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
         // chunk j of the thread is the 24-bit window at bit 24 * j of its bytes: four windows per three dwords
         const int g = j / 4 * 3, jj = j % 4;
         uint32_t d0 = r.w[g], d1 = r.w[g + 1], d2 = W_CH == 2 ? 0u : r.w[W_CH == 2 ? g : g + 2];
-        if (W_CH == 2) {  // the thread's six bytes start at bit 0 or 16 of its two dwords
+        if (W_CH == 2) {  // the thread's six bytes start at bit 0 (even w_part = even lane) or 16 of its two dwords
+          const uint32_t w_sh = (opaque(lane) & 1u) << 4;  // recomputed here: the kernel is at the register limit
           d0 = __builtin_amdgcn_alignbit(d1, d0, w_sh);
           d1 = d1 >> w_sh;
         }
@@ -586,10 +586,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
         // back writes the values the group before it writes, to the same places
         const uint32_t row0 = m0 + wm * 64 + i * 32 + 8 * (e / 4), last = p.M >= 8 ? p.M - 8 : 0;
         const uint32_t m = (row0 < last ? row0 : last) + 4 * (ln >> 5) + (e % 4);
-        if (row0 < p.M && m < p.M && n < p.N) {
-          if (p.out_f32) reinterpret_cast<float*>(p.out)[(size_t)m * p.N + n] = tot[i][j][e];
-          else p.out[(size_t)m * p.N + n] = (_Float16)tot[i][j][e];
-        }
+        if (row0 < p.M && m < p.M && n < p.N) p.out[(size_t)m * p.N + n] = (_Float16)tot[i][j][e];
       }
     }
 }
@@ -617,10 +614,10 @@ hipError_t launch_tile(GemmParams p, bool affine, uint32_t bits, hipStream_t s) 
 }
 
 }  // namespace
-// 4-bit (affine or symmetric), 8-bit or 3-bit affine, f16 or f32 output, dense, K a multiple of 64.
+// 4-bit (affine or symmetric), 8-bit or 3-bit affine, f16 output, dense, K a multiple of 64.
 // The scales are fetched as 4-byte pairs, so a row of them must start on 4 bytes.
 bool gemm_supports(const MatmulArgs& a) {
-  return a.slots == 0 && (a.bits == 4 || ((a.bits == 8 || a.bits == 3) && a.affine)) && a.K % KS == 0 && a.spr % 2 == 0;
+  return a.slots == 0 && (a.bits == 4 || ((a.bits == 8 || a.bits == 3) && a.affine)) && !a.out_f32 && a.K % KS == 0 && a.spr % 2 == 0;
 }
 
 static uint32_t xs_stride_of(const MatmulArgs& a) { return (2 * a.spr + KS - 1) / KS * KS; }
@@ -637,7 +634,6 @@ hipError_t launch_gemm(const MatmulArgs& a, const Tune& t, void* scratch, hipStr
   p.xs_stride = xs_stride_of(a);
   p.bias_steps = a.affine ? p.xs_stride / KS : 0;
   p.xcd_swizzle = t.gemm_xcd_swizzle;
-  p.out_f32 = a.out_f32 ? 1u : 0u;
   if (a.affine) {
     const uint32_t pad = p.xs_stride - 2 * a.spr, cpr = a.K / 8;
     const uint32_t n = a.M * (cpr > pad ? cpr : pad);  // one thread per chunk, and enough for the padding columns
