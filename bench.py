@@ -65,15 +65,17 @@ def timed_graph(ctx, launches, reps=1, warm=1):
     for fn in launches:
         fn()
     cb = ctx.record_end()
+    # one replay in flight at a time: each is waited for before the next is submitted
     for _ in range(warm):
         ctx.submit(cb)
-    ctx.sync()
+        ctx.sync()
     e0, e1 = ctx.event(), ctx.event()
-    ctx.event_record(e0)
+    ms = 0.0
     for _ in range(reps):
+        ctx.event_record(e0)
         ctx.submit(cb)
-    ctx.event_record(e1)
-    ms = ctx.elapsed_ms(e0, e1)
+        ctx.event_record(e1)
+        ms += ctx.elapsed_ms(e0, e1)
     ctx.event_destroy(e0)
     ctx.event_destroy(e1)
     ctx.cmdbuf_destroy(cb)
