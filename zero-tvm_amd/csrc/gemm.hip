@@ -378,14 +378,35 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
       for (int e = 0; e < 16; e++) tot[i][j][e] = 0.f;
   const f16v zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 
-  // ---- bias term first (affine): tot = [xs_hi | xs_lo] x biases on the matrix cores, 64 columns
-  // per step, stage 0 only, no overlap (two or three short steps).
+  // ---- the pipeline's first fetches go out before anything else: the activations of steps 0 and 1 into stages 0
+  // and 1, the packed words of steps 0, 1 and 2 into registers, scale batch 0 into the ring. They land while the
+  // bias term below is computed (through stage 2, which the pipeline does not touch before its first step).
+  const uint32_t nsteps = p.nsteps;
+  WRegs wcur, wnext, w_first;
+  if (sc_loader) load_sc(0);
+  auto load_a = [&](uint32_t stage) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < A_LOADS; i++) {
+      dma16(a_base[i], a_lane, lds_slot(stage, i));
+      a_base[i] += KS;
+    }
+  };
+  load_a(0);
+  load_w(w_first);
+  if (nsteps > 1) {
+    load_a(1);
+    load_w(wnext);
+  }
+  if (nsteps > 2) load_w(wcur);
+
+  // ---- bias term (affine): tot = [xs_hi | xs_lo] x biases on the matrix cores, 64 columns per step, through
+  // stage 2 (two or three short steps).
   if (AFFINE) {
     const uint32_t G = p.spr;
     const _Float16* brow = p.biases + (size_t)w_n * G;
     for (uint32_t bs = 0; bs < p.bias_steps; bs++) {
 #pragma unroll
-      for (int i = 0; i < A_LOADS; i++) dma16(p.xs16 + (size_t)a_row0[i] * p.xs_stride + bs * KS, xs_lane, lds_slot(0, i));
+      for (int i = 0; i < A_LOADS; i++) dma16(p.xs16 + (size_t)a_row0[i] * p.xs_stride + bs * KS, xs_lane, lds_slot(2, i));
 #pragma unroll
       for (int j = 0; j < W_CH; j++) {
         const uint32_t col = bs * KS + (w_part * W_CH + j) * 8;  // column c meets b[n][c mod G]; zero past 2G
@@ -399,7 +420,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
               if (col + e < 2 * G) v[e] = brow[(col + e) % G];
           }
         }
-        *reinterpret_cast<h8*>(smem + w_dst[j]) = v;
+        *reinterpret_cast<h8*>(smem + 2 * STAGE_BYTES + w_dst[j]) = v;
       }
       __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
       __syncthreads();
@@ -407,9 +428,9 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
       for (int ks = 0; ks < KS / 16; ks++) {
         h8 af[2], bf[2];
 #pragma unroll
-        for (int i = 0; i < 2; i++) af[i] = read_a(0, i, ks);
+        for (int i = 0; i < 2; i++) af[i] = read_a(2, i, ks);
 #pragma unroll
-        for (int j = 0; j < 2; j++) bf[j] = read_b(0, j, ks);
+        for (int j = 0; j < 2; j++) bf[j] = read_b(2, j, ks);
 #pragma unroll
         for (int i = 0; i < 2; i++)
 #pragma unroll
@@ -428,27 +449,11 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
   h8 Bf[2][KS / 16], Aq[4];
   f16v part[2][2];
   float sc[SCALES][2], scp[2];  // scales of this step; of the last group of the previous step
-  WRegs wcur, wnext;
 
-  const uint32_t nsteps = p.nsteps;
-  // prologue: stages 0 and 1 complete, weights of step 2 in registers, scale batch 0 in the ring
-  if (sc_loader) load_sc(0);
-  auto load_a = [&](uint32_t stage) __attribute__((always_inline)) {
-#pragma unroll
-    for (int i = 0; i < A_LOADS; i++) {
-      dma16(a_base[i], a_lane, lds_slot(stage, i));
-      a_base[i] += KS;
-    }
-  };
-  load_a(0);
-  load_w(wcur);
-  store_w_words(wcur, 0, 0, W_CH);
-  if (nsteps > 1) {
-    load_a(1);
-    load_w(wcur);
-    store_w_words(wcur, 1, 0, W_CH);
-  }
-  if (nsteps > 2) load_w(wcur);
+  // stages 0 and 1 complete, weights of step 2 in registers, scale batch 0 in the ring
+  __builtin_amdgcn_s_waitcnt(0x0070);
+  store_w_words(w_first, 0, 0, W_CH);
+  if (nsteps > 1) store_w_words(wnext, 1, 0, W_CH);
   __builtin_amdgcn_s_waitcnt(0x0070);
   __syncthreads();
   static_for<4>([&](auto pc) {
