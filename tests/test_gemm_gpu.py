@@ -36,7 +36,8 @@ def make(synth, affine, CAP, N, K, regime="A"):
 
 
 CASES = [(6, 8, 64, 2560, False), (31, 64, 256, 2560, True), (47, 64, 200, 2560, False), (47, 64, 200, 2560, True),
-         (13, 64, 96, 128, True), (13, 64, 96, 128, False), (130, 256, 136, 512, True), (300, 320, 264, 1024, True)]
+         (13, 64, 96, 128, True), (13, 64, 96, 128, False), (130, 256, 136, 512, True), (300, 320, 264, 1024, True),
+         (200, 200, 72, 64, False), (270, 272, 72, 192, False)]  # one and three k steps: no hot loop, short pipelines
 
 
 @pytest.mark.parametrize("M,CAP,N,K,affine", CASES)
