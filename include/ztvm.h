@@ -30,7 +30,11 @@
 extern "C" {
 #endif
 
-#define ZTVM_ABI_VERSION 1
+#define ZTVM_ABI_VERSION 2
+
+/* ztvm_matmul_desc.experts: the caller vouches for every id in ids[] */
+#define ZTVM_EXPERTS_UNCHECKED 0xFFFFFFFFu
+
 
 #if defined(__GNUC__)
 #define ZTVM_API __attribute__((visibility("default")))
@@ -79,8 +83,11 @@ typedef struct ztvm_event ztvm_event;
  * weights/scales/biases are [experts][N][...] stacks, the input row starts at
  * element token*in_tok_stride + slot*in_slot_stride of `in` and the output
  * row at token*out_tok_stride + slot*out_slot_stride of `out`
- * (:236-253). A pair whose expert id is >= experts (when experts != 0) is
- * skipped, so a bad id cannot fault the GPU. */
+ * (:236-253). `experts` is the height of the bound stacks (WebGPU bounds-checks
+ * storage accesses against the bound sizes; here the kernel checks the id): a
+ * pair whose expert id is >= experts is skipped, so a bad id cannot fault the
+ * GPU. A MoE descriptor with experts == 0 is rejected; a caller that has
+ * validated its ids itself passes ZTVM_EXPERTS_UNCHECKED. */
 typedef struct ztvm_matmul_desc {
   uint32_t bits;           /* 4 | 3 */
   uint32_t affine;         /* 0 | 1 */
@@ -97,7 +104,7 @@ typedef struct ztvm_matmul_desc {
   uint32_t in_tok_stride;
   uint32_t out_tok_stride;
   uint32_t ids_stride;
-  uint32_t experts;        /* stack height for the id guard; 0 = unchecked */
+  uint32_t experts;        /* MoE: stack height for the id guard (or ZTVM_EXPERTS_UNCHECKED); ignored when dense */
   uint64_t out;            /* binding 0 (device address incl. region offset) */
   uint64_t in;             /* binding 1 */
   uint64_t scales;         /* binding 2 */
@@ -155,6 +162,14 @@ ZTVM_API int ztvm_matmul_resolve(const ztvm_matmul_desc* desc);
  * :2151-2179; call sites :2290, :2312, :2343-2347, :2517-2524, :2543-2549,
  * :4280-4293, :4386-4390). Validates, then enqueues. */
 ZTVM_API int ztvm_matmul(ztvm_ctx* ctx, const ztvm_matmul_desc* desc);
+
+/* Library-owned scratch. The rows, skinny and tile-GEMM families keep activation group sums,
+ * reordered activations and split-k partial sums in a buffer the context owns (4 MiB at first). A
+ * dispatch that needs more grows it, outside a recording only (inside one the call returns
+ * ZTVM_E_UNSUPPORTED and asks for one eager dispatch of that shape first). Growing never frees a
+ * buffer that a live command buffer may reference: it is kept until the last such command buffer
+ * is destroyed, so a command buffer recorded earlier stays valid to submit after any later
+ * dispatch. Destroying the context ends the life of its command buffers. */
 
 /* Gate + up + SiLU in one pass over the activations: out[n] = up[n] * silu(gate[n]) with
  * gate = W_gate x (the descriptor's weights / scales / biases) and up = W_up x (the three

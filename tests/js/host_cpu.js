@@ -5,7 +5,7 @@ const assert = require('assert')
 const path = require('path')
 const z = require(path.join(__dirname, '..', '..', 'zero-tvm_amd', 'js'))
 
-assert.strictEqual(z.abiVersion(), 1)
+assert.strictEqual(z.abiVersion(), 2)
 const names = z.INT4_MATMUL_VARIANTS.map(z.int4MatmulEntry)
 assert.strictEqual(names.length, 34)
 assert.strictEqual(new Set(names).size, 34)

@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol(capi):
     for n in names:
         assert hasattr(lib, n), n
     assert sorted(capi.EXPORTS) == names
-    assert lib.ztvm_abi_version() == 1
+    assert lib.ztvm_abi_version() == 2
 
 
 def test_desc_struct_matches_header_layout(capi):
@@ -72,6 +72,7 @@ def test_validator_accepts_reference_shapes(capi):
     (dict(slots=8, tokens=2, ids=0x6000, ids_stride=8, M=4, out_slot_stride=64), "M must be 1"),
     (dict(slots=8, tokens=2, ids=0x6000, ids_stride=8, in_slot_stride=4, out_slot_stride=64), "multiples of 8"),
     (dict(slots=8, tokens=2, ids=0x6000, ids_stride=8, out_slot_stride=8), "overlap"),
+    (dict(slots=8, tokens=2, ids=0x6000, ids_stride=8, out_slot_stride=64), "experts"),   # the id guard must be armed
     (dict(kernel=9), "kernel"),
     (dict(N=1 << 20), "2 GiB"),                            # 2^20 rows of 512 words = 2 GiB: 32-bit byte offsets end here
 ])
@@ -83,7 +84,7 @@ def test_validator_rejects(capi, kw, needle):
 def test_explicit_kernel_that_cannot_run_is_an_error(capi):
     """Never a silent substitution (pickChunkGemm, src/zero-tvm/engine-core.ts:220-245)."""
     moe = good(capi, N=512, k_packed=256, scales_per_row=32, slots=8, tokens=1, out_slot_stride=512, ids_stride=8,
-               ids=0x6000, kernel=capi.KERNEL_GEMM)
+               ids=0x6000, experts=256, kernel=capi.KERNEL_GEMM)
     rc, why = capi.validate(moe)
     assert rc == capi.E_UNSUPPORTED and "asked for" in why
     with pytest.raises(capi.ZtvmError):
@@ -104,6 +105,23 @@ def test_auto_picks_a_family_by_rows(capi):
     odd = dict(M=300, k_packed=24, scales_per_row=3)
     assert capi.resolve(good(capi, **odd)) == capi.KERNEL_SKINNY
     assert capi.validate(good(capi, kernel=capi.KERNEL_GEMM, **odd))[0] == capi.E_UNSUPPORTED
+
+
+def test_unchecked_experts_is_an_explicit_choice(capi):
+    moe = dict(N=512, k_packed=256, scales_per_row=32, slots=8, tokens=1, out_slot_stride=512, ids_stride=8, ids=0x6000)
+    assert capi.validate(good(capi, **moe))[0] == capi.E_INVALID
+    assert capi.validate(good(capi, experts=capi.EXPERTS_UNCHECKED, **moe))[0] == 0
+
+
+def test_rows_too_long_for_the_gemv_staging_are_refused(capi):
+    """The GEMV family stages the activation row in LDS (160 KB): a dispatch that has no other family
+    (M = 1 explicit GEMV, MoE) and a longer row is an error before any launch, dense rows go elsewhere."""
+    K = 1 << 17
+    big = dict(k_packed=K // 8, scales_per_row=K // 64, N=64)
+    rc, why = capi.validate(good(capi, kernel=capi.KERNEL_GEMV, **big))
+    assert rc == capi.E_UNSUPPORTED and "LDS" in why, why
+    K = 65536  # 139264 B of staging: fits
+    assert capi.validate(good(capi, kernel=capi.KERNEL_GEMV, k_packed=K // 8, scales_per_row=K // 64, N=64))[0] == 0
 
 
 def test_no_device_is_a_loud_error(capi):

@@ -159,3 +159,28 @@ def test_pod_builders_match_the_engine(eng):
     assert g3[0] == 192 and d3[0] == 48
     assert eng.dense_pod(4096, 14336) == [512, 64, 14336]
     assert eng.dense_pod(4096, 14336, affine=False, M=31) == [512, 128, 14336, 31]
+
+
+def test_moe_descriptor_arms_the_expert_guard(eng, capi):
+    """The engine-built MoE descriptor carries the stack height taken from the bound sizes (what WebGPU's
+    bounds-checked storage access gave the reference), and bound stacks that disagree are refused."""
+    E, d_model, ffn, slots = 6, 256, 128, 3
+    gate, _ = eng.moe_pods(d_model, ffn, slots)
+
+    class FakeBuf:
+        def __init__(self, size):
+            self.addr, self.size = 0x10000, size
+
+    dev = eng.Device.__new__(eng.Device)
+    pipe = eng.create_pipeline("int4_matmul_tiled_affine_moe")
+    per_w, per_s = ffn * (d_model // 8) * 4, ffn * (d_model // 64) * 2
+    bufs = [FakeBuf(slots * 2 * ffn * 2), FakeBuf(d_model * 2), FakeBuf(E * per_s), FakeBuf(E * per_w), dev.uniform_buf(gate),
+            FakeBuf(E * per_s), FakeBuf(slots * 4)]
+    desc = dev.descriptor(dev.bg(pipe, bufs), ffn // 4, 1, slots)
+    assert desc.experts == E and desc.slots == slots and desc.tokens == 1
+    assert capi.validate(desc)[0] == 0
+    bufs[5] = FakeBuf((E - 2) * per_s)             # a bias stack two experts short: the guard takes the smallest
+    assert dev.descriptor(dev.bg(pipe, bufs), ffn // 4, 1, slots).experts == E - 2
+    bufs[3] = FakeBuf(per_w - 4)                   # not even one whole expert bound
+    with pytest.raises(ValueError, match="no whole expert"):
+        dev.descriptor(dev.bg(pipe, bufs), ffn // 4, 1, slots)

@@ -8,7 +8,7 @@ import importlib
 import numpy as np
 import pytest
 
-from .util import Dev
+from .util import Dev, rel_err
 
 pytestmark = pytest.mark.gpu
 
@@ -48,7 +48,7 @@ def gate_desc(capi, N, K, S, ids, x, out, w, s, b, experts):
 
 
 @pytest.mark.parametrize("optimistic", [False, True])
-def test_pooled_equals_full_stack(ctx, capi, synth, ep, device, optimistic):
+def test_pooled_equals_full_stack(ctx, capi, synth, oracle, ep, device, optimistic):
     d, ffn, E, K, SLOTS = 256, 128, 24, 4, 8
     E1, S = E + 1, K + 1                       # a shared expert at index E, pinned
     st = stacks(synth, E1, d, ffn)
@@ -64,12 +64,18 @@ def test_pooled_equals_full_stack(ctx, capi, synth, ep, device, optimistic):
             out_f, out_p = dv.empty(S * ffn * 2, fill=0), dv.empty(S * ffn * 2, fill=0)
             for step in range(40):
                 experts = np.r_[rng.choice(E, K, replace=False), E].astype(np.uint32)
-                x = dv.put(synth.activations(1, d, salt=step))
+                xh = synth.activations(1, d, salt=step)
+                x = dv.put(xh)
                 ctx.upload(ids_e, experts)
                 for proj in ("gate", "up"):
                     w, s, b = full[proj]
                     ctx.matmul(gate_desc(capi, ffn, d, S, ids_e, x, out_f, w, s, b, E1))
                     want = ctx.download(out_f, S * ffn * 2, np.uint16)
+                    if step % 8 == 0:
+                        # the full-stack result itself against the oracle: "pooled == full" alone would pass a shared error
+                        ref = oracle.moe_gemv(oracle.MODE_FORMULA_F32, 4, ffn, d, 1, S, (0, ffn, d, S * ffn, S), experts, xh,
+                                              *st[proj], S * ffn, threads=4)
+                        assert rel_err(want.view(np.float16).astype(np.float64), ref, 1e-2) < 1e-2, (step, proj)
                     bufs = lp.buffers
                     pw, ps, pb = (bufs[proj + "Weights"].addr, bufs[proj + "Scales"].addr, bufs[proj + "Biases"].addr)
                     if optimistic:

@@ -168,13 +168,13 @@ def test_rows_past_the_last_full_group(ctx, capi, synth, oracle, rows):
     assert np.array_equal(got[:rows], full[:rows]), "a row depends on how many rows follow it"
 
 
-@pytest.mark.parametrize("M", [128, 512])
+@pytest.mark.parametrize("M", [128, 512, 2048])
 def test_config3_shape(ctx, capi, synth, oracle, M):
     """configs[2]: K=4096, N=14336; checked on a row sample against the formula and the f16-weight reference."""
     K, N = 4096, 14336
     A, w, s, b = make(synth, True, M, N, K)
     got = run(ctx, capi, True, M, M, N, K, A, w, s, b, capi.KERNEL_GEMM)
-    rows = np.array([0, 1, M // 2, M - 1])
+    rows = np.array([0, 1, M // 2, M - 1])   # first and last tile row of the grid (M=2048: 8 tile rows, 3.5 rounds of workgroups)
     y = got[rows].view(np.float16).astype(np.float64)
     ref = oracle.gemm(oracle.MODE_FORMULA_F64, 4, True, len(rows), N, K, A[rows], w, s, b, threads=8)
     e = rel_err(y, ref, 1e-2)
@@ -183,3 +183,43 @@ def test_config3_shape(ctx, capi, synth, oracle, M):
     # every row agrees with the GEMV family's answer for the same row (two independent kernels)
     gv = run(ctx, capi, True, 4, 4, N, K, A[rows], w, s, b, capi.KERNEL_GEMV)
     assert rel_err(y, gv.view(np.float16).astype(np.float64), 1e-2) < 1e-2
+
+
+def test_recorded_gemm_survives_scratch_growth(ctx, capi, synth, oracle):
+    """A command buffer keeps the scratch address of its GEMM (activation group sums). A later eager
+    dispatch that needs more scratch than the context owns must not free what the command buffer
+    references: record, grow, replay, and the replay still equals the eager result and the oracle."""
+    M, N, K = 160, 136, 512
+    A, w, s, b = make(synth, True, M, N, K)
+    eager = run(ctx, capi, True, M, M, N, K, A, w, s, b, capi.KERNEL_GEMM)
+    with Dev(ctx) as d:
+        out = d.empty(M * N * 2, fill=0)
+        desc = capi.MatmulDesc(bits=4, affine=1, kernel=capi.KERNEL_GEMM, M=M, N=N, k_packed=K // 8, scales_per_row=K // 64,
+                               out=out, in_=d.put(A), scales=d.put(s), weights=d.put(w), biases=d.put(b))
+        ctx.record_begin()
+        ctx.matmul(desc)
+        cb = ctx.record_end()
+        try:
+            ctx.submit(cb)
+            first = ctx.download(out, M * N * 2, np.uint16).reshape(M, N)
+            assert np.array_equal(first, eager)
+            # a skinny dispatch whose f32 partial sums outgrow any scratch this session has allocated so far
+            Mb, Nb, Kb = 128, 40960, 256
+            big = capi.MatmulDesc(bits=4, affine=1, kernel=capi.KERNEL_SKINNY, M=Mb, N=Nb, k_packed=Kb // 8, scales_per_row=Kb // 64,
+                                  out=d.empty(Mb * Nb * 2), in_=d.put(synth.activations(Mb, Kb)), scales=d.put(synth.scales(Nb, Kb)),
+                                  weights=d.put(synth.packed_weights(Nb, Kb)), biases=d.put(synth.biases(Nb, Kb, synth.scales(Nb, Kb))))
+            ctx.set_option("skinny.ksplit", 4)   # 4 x 128 x 40960 f32 partial sums = 80 MiB
+            try:
+                ctx.matmul(big)
+                ctx.sync()
+            finally:
+                ctx.set_option("skinny.ksplit", 0)
+            for _ in range(2):
+                ctx.fill(out, 0, M * N * 2)
+                ctx.submit(cb)
+                again = ctx.download(out, M * N * 2, np.uint16).reshape(M, N)
+                assert np.array_equal(again, eager), "replay after the scratch grew differs from the eager result"
+        finally:
+            ctx.cmdbuf_destroy(cb)
+    ref = oracle.gemm(oracle.MODE_FORMULA_F64, 4, True, M, N, K, A, w, s, b, threads=8)
+    assert rel_err(eager.view(np.float16).astype(np.float64), ref, 1e-2) < 1e-2

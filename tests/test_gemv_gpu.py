@@ -136,3 +136,30 @@ def test_seeded_random_shapes(ctx, capi, synth, oracle):
         err = rel_err(y, ref, 1e-2)
         assert err < 1e-2, (case, bits, affine, N, K, err)
         assert not raw[N * esz:].any(), "wrote past N"
+
+
+@pytest.mark.parametrize("regime", ["A", "B"])
+def test_gate_sees_a_wrong_kernel(ctx, capi, synth, oracle, regime):
+    """configs[0] through the GPU against references computed from deliberately wrong inputs (the mutations of
+    scripts/mutation-gate.mjs): the GPU result passes the gate against the right reference and FAILS it against a
+    reference with a shifted scale group, a dropped bias or a swapped nibble order — the 1e-2 bar with its 1e-2
+    floor in the denominator is tight enough to tell them apart."""
+    from .util import mutations
+    K, N = 2048, 8192
+    x, w, s = synth.activations(1, K), synth.packed_weights(N, K), synth.scales(N, K)
+    b = synth.biases(N, K, s, regime)
+    y = run_dense(ctx, capi, 4, True, 1, N, K, x, w, s, b)
+    check(y, oracle, 4, True, 1, N, K, x, w, s, b)
+    for name, (mw, ms, mb) in mutations(w, s, b).items():
+        wrong = oracle.gemm(oracle.MODE_FORMULA_F32, 4, True, 1, N, K, x, mw, ms, mb, threads=8)
+        assert rel_err(y, wrong, 1e-2) > 10 * 1e-2, name
+        assert np.median(np.abs(y - wrong) / (np.abs(wrong) + 1e-2)) > 1e-2, name
+
+
+def test_long_rows_k32768(ctx, capi, synth, oracle):
+    """K = 32768: 68 KB of staged activations, past the 64 KB a launch gets without asking for more."""
+    K, N = 32768, 96
+    x, w, s = synth.activations(1, K), synth.packed_weights(N, K), synth.scales(N, K)
+    b = synth.biases(N, K, s)
+    y = run_dense(ctx, capi, 4, True, 1, N, K, x, w, s, b, kernel=capi.KERNEL_GEMV)
+    check(y, oracle, 4, True, 1, N, K, x, w, s, b)

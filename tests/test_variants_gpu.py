@@ -100,7 +100,6 @@ def test_moe_block_config4(ctx, capi, synth, oracle, tokens, bits):
                               got.size, threads=8)
         refu = oracle.moe_gemv(oracle.MODE_FORMULA_F32, bits, ffn, d_model, tokens, slots, strides, ids, x, wu, sg, bg,
                                got.size + ffn, threads=8)
-        ref[ffn:] += refu[:-ffn][: ref.size - ffn] * 0  # keep shapes; the up half is compared below
         g3 = got.reshape(tokens, slots, 2, ffn)
         assert rel_err(g3[:, :, 0], ref.reshape(tokens, slots, 2, ffn)[:, :, 0], 1e-2) < 1e-2
         assert rel_err(g3[:, :, 1], refu[: got.size].reshape(tokens, slots, 2, ffn)[:, :, 0], 1e-2) < 1e-2

@@ -43,3 +43,16 @@ def rel_err(got, ref, eps):
 
 def f16(bits):
     return np.asarray(bits, np.uint16).view(np.float16).astype(np.float64)
+
+
+def mutations(w, s, b):
+    """The wrong kernels of the reference's mutation gate (scripts/mutation-gate.mjs; its figures at
+    BENCH.md:1694-1701: unshifted scale index 2.51e+0, dropped bias 1.95e-1), expressed as wrong INPUTS to a
+    correct reference: name -> (weights, scales, biases). A parity gate that passes any of them sees nothing."""
+    w, s, b = np.asarray(w), np.asarray(s), np.asarray(b)
+    swapped = ((w & np.uint32(0x0F0F0F0F)) << np.uint32(4)) | ((w >> np.uint32(4)) & np.uint32(0x0F0F0F0F))
+    return {
+        "scale group shifted by one": (w, np.roll(s, 1, axis=-1), b),
+        "bias dropped": (w, s, np.zeros_like(b)),
+        "nibble order swapped": (swapped.astype(np.uint32), s, b),
+    }

@@ -380,34 +380,41 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(const GemvParams p) {
   }
 }
 
+// Launch with `smem` bytes of dynamic LDS; above 64 KB the kernel's limit has to be raised first.
+template <class Kernel>
+void go(Kernel k, dim3 grid, uint32_t threads, size_t smem, hipStream_t s, const GemvParams& p) {
+  if (smem > 64 * 1024) (void)hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+  hipLaunchKernelGGL(k, grid, dim3(threads), smem, s, p);
+}
+
 template <int BITS, bool AFFINE, int LPR, int ROWS>
 hipError_t launch_one(const GemvParams& p, dim3 grid, uint32_t threads, size_t smem, hipStream_t s) {
-  if (threads > 512) hipLaunchKernelGGL((gemv_kernel<BITS, AFFINE, LPR, ROWS, 1024>), grid, dim3(threads), smem, s, p);
-  else hipLaunchKernelGGL((gemv_kernel<BITS, AFFINE, LPR, ROWS, 512>), grid, dim3(threads), smem, s, p);
+  if (threads > 512) go(gemv_kernel<BITS, AFFINE, LPR, ROWS, 1024>, grid, threads, smem, s, p);
+  else go(gemv_kernel<BITS, AFFINE, LPR, ROWS, 512>, grid, threads, smem, s, p);
   return hipGetLastError();
 }
 
 template <int BITS, bool AFFINE>
 hipError_t launch_qkv(const GemvParams& p, int lpr, dim3 grid, uint32_t threads, size_t smem, hipStream_t s) {
-  if (lpr == 64) hipLaunchKernelGGL((gemv_kernel<BITS, AFFINE, 64, 1, 512, true, true>), grid, dim3(threads), smem, s, p);
-  else if (lpr == 32) hipLaunchKernelGGL((gemv_kernel<BITS, AFFINE, 32, 1, 512, true, true>), grid, dim3(threads), smem, s, p);
-  else hipLaunchKernelGGL((gemv_kernel<BITS, AFFINE, 16, 1, 512, true, true>), grid, dim3(threads), smem, s, p);
+  if (lpr == 64) go(gemv_kernel<BITS, AFFINE, 64, 1, 512, true, true>, grid, threads, smem, s, p);
+  else if (lpr == 32) go(gemv_kernel<BITS, AFFINE, 32, 1, 512, true, true>, grid, threads, smem, s, p);
+  else go(gemv_kernel<BITS, AFFINE, 16, 1, 512, true, true>, grid, threads, smem, s, p);
   return hipGetLastError();
 }
 
 template <int BITS, bool AFFINE>
 hipError_t launch_prologue(const GemvParams& p, int lpr, dim3 grid, uint32_t threads, size_t smem, hipStream_t s) {
-  if (lpr == 64) hipLaunchKernelGGL((gemv_kernel<BITS, AFFINE, 64, 1, 512, true, false, true>), grid, dim3(threads), smem, s, p);
-  else if (lpr == 32) hipLaunchKernelGGL((gemv_kernel<BITS, AFFINE, 32, 1, 512, true, false, true>), grid, dim3(threads), smem, s, p);
-  else hipLaunchKernelGGL((gemv_kernel<BITS, AFFINE, 16, 1, 512, true, false, true>), grid, dim3(threads), smem, s, p);
+  if (lpr == 64) go(gemv_kernel<BITS, AFFINE, 64, 1, 512, true, false, true>, grid, threads, smem, s, p);
+  else if (lpr == 32) go(gemv_kernel<BITS, AFFINE, 32, 1, 512, true, false, true>, grid, threads, smem, s, p);
+  else go(gemv_kernel<BITS, AFFINE, 16, 1, 512, true, false, true>, grid, threads, smem, s, p);
   return hipGetLastError();
 }
 
 template <int BITS, bool AFFINE>
 hipError_t launch_gated(const GemvParams& p, int lpr, dim3 grid, uint32_t threads, size_t smem, hipStream_t s) {
-  if (lpr == 64) hipLaunchKernelGGL((gemv_kernel<BITS, AFFINE, 64, 1, 512, true>), grid, dim3(threads), smem, s, p);
-  else if (lpr == 32) hipLaunchKernelGGL((gemv_kernel<BITS, AFFINE, 32, 1, 512, true>), grid, dim3(threads), smem, s, p);
-  else hipLaunchKernelGGL((gemv_kernel<BITS, AFFINE, 16, 1, 512, true>), grid, dim3(threads), smem, s, p);
+  if (lpr == 64) go(gemv_kernel<BITS, AFFINE, 64, 1, 512, true>, grid, threads, smem, s, p);
+  else if (lpr == 32) go(gemv_kernel<BITS, AFFINE, 32, 1, 512, true>, grid, threads, smem, s, p);
+  else go(gemv_kernel<BITS, AFFINE, 16, 1, 512, true>, grid, threads, smem, s, p);
   return hipGetLastError();
 }
 
@@ -422,7 +429,15 @@ hipError_t launch_fmt(const GemvParams& p, int lpr, int rows, dim3 grid, uint32_
   return launch_one<BITS, AFFINE, 16, 2>(p, grid, threads, smem, s);
 }
 
+size_t gemv_lds_bytes(uint32_t K, uint32_t head_dim, bool prologue) {
+  const uint32_t padded_chunks = (K / 32u + 63u) & ~63u;
+  return (size_t)padded_chunks * 68u + (size_t)(head_dim / 2) * 8u + (prologue ? 64u : 0u);
+}
+
 }  // namespace
+
+// The activation row is staged whole in LDS (160 KB per CU).
+bool gemv_supports(const MatmulArgs& a) { return gemv_lds_bytes(a.K, a.qkv ? a.qkv->head_dim : 0, a.delta != nullptr) <= 160u * 1024u; }
 
 hipError_t launch_gemv(const MatmulArgs& a, const Tune& t, hipStream_t s) {
   GemvParams p{};
@@ -458,7 +473,7 @@ hipError_t launch_gemv(const MatmulArgs& a, const Tune& t, hipStream_t s) {
   // workgroups, 3 per CU, stream best for wide rows; narrow rows (several rows
   // per wave load) use 2 steps in flight.
   const int cus = t.num_cus;
-  int rows = lpr == 64 ? (t.gemv_rows ? t.gemv_rows : 1) : 2;
+  int rows = lpr == 64 ? (t.gemv_rows == 2 || t.gemv_rows == 4 ? t.gemv_rows : 1) : 2;
   if (gated) rows = 1;  // two matrices per row already give two loads in flight
   // long rows (K >= 8192): the staged activations are 16+ KB per workgroup, so one 16-wave
   // workgroup per CU stages them once instead of three times (measured 9.4 vs 10.2 us at K=14336)
@@ -470,9 +485,8 @@ hipError_t launch_gemv(const MatmulArgs& a, const Tune& t, hipStream_t s) {
   const uint32_t rpw = rows * (64 / lpr);
   p.ntiles = (a.N + rpw - 1) / rpw;
 
-  const uint32_t padded_chunks = (p.nchunks + 63u) & ~63u;
-  const size_t smem = (size_t)padded_chunks * 64 + (size_t)padded_chunks * 4 + (a.qkv ? (size_t)(a.qkv->head_dim / 2) * 8 : 0) +
-                      (a.delta ? 64 : 0);  // the prologue's per-wave sums of squares
+  if (!gemv_supports(a)) return hipErrorInvalidValue;  // rejected by the entry points
+  const size_t smem = gemv_lds_bytes(a.K, a.qkv ? a.qkv->head_dim : 0, a.delta != nullptr);
 
   const uint32_t wg_tiles = (p.ntiles + waves - 1) / waves;
   gx = gx / pairs;

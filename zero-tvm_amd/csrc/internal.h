@@ -48,9 +48,6 @@ struct Tune {
   int gemv_wg_per_cu = 0;   // workgroups resident per CU for the streaming GEMV
   int gemv_rows = 0;        // rows per wave step (1, 2 or 4)
   int gemv_waves = 0;       // waves per workgroup (4..8)
-  int gemv_path = 0;        // 0/1: the f16 dot2 kernel; 2: the int8 matrix-core kernel (opt-in)
-  int i8_ksplit = 0;        // waves sharing one tile in the int8 GEMV (1, 2 or 4)
-  int i8_wg_per_cu = 0;
   int skinny_ksplit = 0;     // workgroups sharing the k range of one skinny tile (0: chosen from M, N, K)
   int rows_wg_per_cu = 0;    // the row-group GEMV: workgroups per CU and waves per workgroup (0: chosen from the LDS it stages)
   int rows_waves = 0;
@@ -59,8 +56,7 @@ struct Tune {
 };
 
 hipError_t launch_gemv(const MatmulArgs& a, const Tune& t, hipStream_t s);
-hipError_t launch_gemv_i8(const MatmulArgs& a, const Tune& t, hipStream_t s);
-bool gemv_i8_supports(const MatmulArgs& a);
+bool gemv_supports(const MatmulArgs& a);  // the activation row fits the LDS staging
 hipError_t launch_skinny(const MatmulArgs& a, const Tune& t, void* scratch, hipStream_t s);
 size_t skinny_scratch_bytes(const MatmulArgs& a, const Tune& t);
 hipError_t launch_gemm(const MatmulArgs& a, const Tune& t, void* scratch, hipStream_t s);

@@ -3,28 +3,53 @@
 // and the reference interfaces each entry point replaces.
 #include "../../include/ztvm.h"
 #include "internal.h"
+#include "scratch_pool.h"
 
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <memory>
 #include <mutex>
 #include <string>
 
 using namespace ztvm;
+
+namespace {
+// hipMalloc / hipFree on the context's device
+struct DeviceAlloc {
+  int device = 0;
+  void* allocate(size_t bytes) const {
+    void* p = nullptr;
+    if (hipSetDevice(device) != hipSuccess || hipMalloc(&p, bytes) != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    return p;
+  }
+  void release(void* p) const {
+    (void)hipSetDevice(device);
+    (void)hipFree(p);  // waits for the device: nothing in flight still reads the buffer
+  }
+};
+using DevicePool = ScratchPool<DeviceAlloc>;
+}  // namespace
 
 struct ztvm_ctx {
   int device = 0;
   hipStream_t stream = nullptr;
   bool recording = false;
   Tune tune;
-  void* scratch = nullptr;  // group sums of the activations for the GEMM's bias term
-  size_t scratch_bytes = 0;
+  // Library-owned device memory of the rows / skinny / tile-GEMM families (activation group sums,
+  // reordered activations, split-k partial sums). Shared with the command buffers recorded on this
+  // context, which keep its addresses alive (scratch_pool.h).
+  std::shared_ptr<DevicePool> scratch;
   std::string err;
   hipDeviceProp_t prop;
 };
 struct ztvm_cmdbuf {
   hipGraph_t graph = nullptr;
   hipGraphExec_t exec = nullptr;
+  std::shared_ptr<DevicePool> scratch;  // pinned while this command buffer lives
 };
 struct ztvm_event {
   hipEvent_t ev = nullptr;
@@ -92,6 +117,7 @@ int validate(const ztvm_matmul_desc* d, char* why, size_t n, bool need_in_out) {
       if (d->ids & 3u) { why_set(why, n, "ids must be 4-byte aligned"); return ZTVM_E_INVALID; }
       if ((d->in_slot_stride | d->in_tok_stride) & 7u) { why_set(why, n, "moe input strides must be multiples of 8 elements"); return ZTVM_E_INVALID; }
       if (d->out_slot_stride < d->N && d->slots > 1) { why_set(why, n, "OUT_SLOT_STRIDE=%u < N=%u would overlap slot outputs", d->out_slot_stride, d->N); return ZTVM_E_INVALID; }
+      if (!d->experts) { why_set(why, n, "moe needs experts > 0 (the height of the bound stacks, which arms the expert-id guard), or ZTVM_EXPERTS_UNCHECKED"); return ZTVM_E_INVALID; }
     } else {
       if (!d->M) { why_set(why, n, "M must be > 0"); return ZTVM_E_INVALID; }
     }
@@ -130,7 +156,18 @@ MatmulArgs to_args(const ztvm_matmul_desc* d) {
 // MI355X: the GEMV re-reads the weights once per activation row, the skinny
 // kernel streams them once through registers for tiles of up to 128 rows, the
 // tile GEMM needs enough rows to fill its 256-row tile.
+int resolve_family(const MatmulArgs& a, uint32_t want, char* why, size_t n);
+
 int resolve(const MatmulArgs& a, uint32_t want, char* why, size_t n) {
+  const int fam = resolve_family(a, want, why, n);
+  if (fam == ZTVM_KERNEL_GEMV && !gemv_supports(a)) {
+    why_set(why, n, "kernel: the GEMV family stages the activation row in LDS and K=%u does not fit (this dispatch has no other family: moe=%d, M=%u)", a.K, (int)(a.slots > 0), a.M);
+    return ZTVM_E_UNSUPPORTED;
+  }
+  return fam;
+}
+
+int resolve_family(const MatmulArgs& a, uint32_t want, char* why, size_t n) {
   const bool moe = a.slots > 0;
   const bool sk = !moe && skinny_supports(a);
   const bool ge = !moe && gemm_supports(a);
@@ -156,6 +193,22 @@ int resolve(const MatmulArgs& a, uint32_t want, char* why, size_t n) {
   return ZTVM_KERNEL_GEMV;
 }
 
+// The context's scratch buffer, grown to `need` bytes if it is smaller. Growing allocates, which a
+// recording cannot hold; outside a recording the old buffer is retired, not freed, while any
+// command buffer that may carry its address is alive.
+int scratch_for(ztvm_ctx* ctx, size_t need, void** out) {
+  DevicePool& pool = *ctx->scratch;
+  if (need > pool.bytes()) {
+    if (ctx->recording)
+      return fail(ctx, ZTVM_E_UNSUPPORTED, "this dispatch needs %zu bytes of scratch (have %zu) and a recording cannot allocate; dispatch it once outside a recording first", need, pool.bytes());
+    hipError_t e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) return fail(ctx, ZTVM_E_HIP, "hipStreamSynchronize: %s", hipGetErrorString(e));
+    if (!pool.reserve(need)) return fail(ctx, ZTVM_E_HIP, "no device memory for %zu bytes of scratch", need);
+  }
+  *out = pool.data();
+  return ZTVM_OK;
+}
+
 struct Option {
   const char* name;
   int Tune::*field;
@@ -165,9 +218,6 @@ const Option kOptions[] = {
     {"gemv.wg_per_cu", &Tune::gemv_wg_per_cu},
     {"gemv.rows", &Tune::gemv_rows},
     {"gemv.waves", &Tune::gemv_waves},
-    {"gemv.path", &Tune::gemv_path},
-    {"i8.ksplit", &Tune::i8_ksplit},
-    {"i8.wg_per_cu", &Tune::i8_wg_per_cu},
     {"skinny.ksplit", &Tune::skinny_ksplit},
     {"rows.wg_per_cu", &Tune::rows_wg_per_cu},
     {"rows.waves", &Tune::rows_waves},
@@ -200,8 +250,12 @@ int ztvm_create(int device, ztvm_ctx** out) {
   }
   HIP_TRY(nullptr, hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
   c->tune.num_cus = c->prop.multiProcessorCount > 0 ? c->prop.multiProcessorCount : 256;
-  c->scratch_bytes = 4u << 20;
-  HIP_TRY(nullptr, hipMalloc(&c->scratch, c->scratch_bytes));
+  c->scratch = std::make_shared<DevicePool>(DeviceAlloc{device});
+  if (!c->scratch->reserve(4u << 20)) {
+    (void)hipStreamDestroy(c->stream);
+    delete c;
+    return fail(nullptr, ZTVM_E_HIP, "ztvm_create: no device memory for the scratch buffer");
+  }
   *out = c;
   return ZTVM_OK;
 }
@@ -213,7 +267,7 @@ void ztvm_destroy(ztvm_ctx* ctx) {
     (void)hipStreamSynchronize(ctx->stream);
     (void)hipStreamDestroy(ctx->stream);
   }
-  if (ctx->scratch) (void)hipFree(ctx->scratch);
+  if (ctx->scratch) ctx->scratch->release_all();  // command buffers of this context are dead with it
   delete ctx;
 }
 
@@ -316,44 +370,24 @@ int ztvm_matmul(ztvm_ctx* ctx, const ztvm_matmul_desc* desc) {
     case ZTVM_KERNEL_SKINNY:
     case ZTVM_KERNEL_GEMM: {
       const size_t need = fam == ZTVM_KERNEL_GEMM ? gemm_scratch_bytes(a) : (fam == ZTVM_KERNEL_ROWS ? rows_scratch_bytes(a) : skinny_scratch_bytes(a, ctx->tune));
-      if (need > ctx->scratch_bytes) {
-        // growing means a free + malloc, which a command buffer cannot hold
-        if (ctx->recording)
-          return fail(ctx, ZTVM_E_UNSUPPORTED, "ztvm_matmul: this dispatch needs %zu bytes of scratch (have %zu); dispatch it once outside a recording first", need, ctx->scratch_bytes);
-        HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
-        HIP_TRY(ctx, hipFree(ctx->scratch));
-        ctx->scratch = nullptr;
-        ctx->scratch_bytes = 0;
-        HIP_TRY(ctx, hipMalloc(&ctx->scratch, need));
-        ctx->scratch_bytes = need;
-      }
-      if (fam == ZTVM_KERNEL_GEMM) HIP_TRY(ctx, launch_gemm(a, ctx->tune, ctx->scratch, ctx->stream));
-      else if (fam == ZTVM_KERNEL_ROWS) HIP_TRY(ctx, launch_rows(a, ctx->tune, ctx->scratch, ctx->stream));
-      else HIP_TRY(ctx, launch_skinny(a, ctx->tune, ctx->scratch, ctx->stream));
+      void* scratch = nullptr;
+      rc = scratch_for(ctx, need, &scratch);
+      if (rc) return rc;
+      if (fam == ZTVM_KERNEL_GEMM) HIP_TRY(ctx, launch_gemm(a, ctx->tune, scratch, ctx->stream));
+      else if (fam == ZTVM_KERNEL_ROWS) HIP_TRY(ctx, launch_rows(a, ctx->tune, scratch, ctx->stream));
+      else HIP_TRY(ctx, launch_skinny(a, ctx->tune, scratch, ctx->stream));
       break;
     }
     default: {
-      // streaming passes over the weights: up to four activation rows per pass on
-      // the int8 matrix-core kernel, one row per pass on the f16 dot2 kernel
+      // one streaming pass over the weights per activation row
       const uint32_t M = a.slots ? 1 : a.M;
       const size_t out_elt = a.out_f32 ? 4 : 2;
-      uint32_t m = 0;
-      while (m < M) {
+      for (uint32_t m = 0; m < M; m++) {
         MatmulArgs r = a;
         r.in = a.in + (size_t)m * a.K;
         r.out = reinterpret_cast<char*>(a.out) + (size_t)m * a.N * out_elt;
-        r.M = a.slots ? 1 : (M - m < 4 ? M - m : 4);
-        const bool i8 = ctx->tune.gemv_path == 2 && gemv_i8_supports(r);
-        if (ctx->tune.gemv_path == 2 && !i8)
-          return fail(ctx, ZTVM_E_UNSUPPORTED, "ztvm_matmul: gemv.path=2 asks for the int8 kernel, which cannot run this dispatch (bits=%u, K=%u)", a.bits, a.K);
-        if (i8) {
-          HIP_TRY(ctx, launch_gemv_i8(r, ctx->tune, ctx->stream));
-          m += r.M;
-        } else {
-          r.M = 1;
-          HIP_TRY(ctx, launch_gemv(r, ctx->tune, ctx->stream));
-          m += 1;
-        }
+        r.M = 1;
+        HIP_TRY(ctx, launch_gemv(r, ctx->tune, ctx->stream));
       }
     }
   }
@@ -374,6 +408,7 @@ int ztvm_ffn_gated(ztvm_ctx* ctx, const ztvm_matmul_desc* desc, uint64_t up_weig
   a.up_weights = reinterpret_cast<const uint32_t*>(up_weights);
   a.up_scales = reinterpret_cast<const _Float16*>(up_scales);
   a.up_biases = reinterpret_cast<const _Float16*>(up_biases);
+  if (!gemv_supports(a)) return fail(ctx, ZTVM_E_UNSUPPORTED, "ztvm_ffn_gated: K=%u does not fit the LDS staging of the activation row", a.K);
   const uint32_t M = a.slots ? 1 : a.M;
   const size_t out_elt = a.out_f32 ? 4 : 2;
   for (uint32_t m = 0; m < M; m++) {  // one pass over both matrices per activation row
@@ -407,6 +442,7 @@ int ztvm_ffn_gated_prologue(ztvm_ctx* ctx, const ztvm_matmul_desc* desc, uint64_
   a.delta = reinterpret_cast<const _Float16*>(delta);
   a.gamma = reinterpret_cast<const _Float16*>(gamma);
   a.rms_eps = rms_eps;
+  if (!gemv_supports(a)) return fail(ctx, ZTVM_E_UNSUPPORTED, "ztvm_ffn_gated_prologue: K=%u does not fit the LDS staging of the activation row", a.K);
   HIP_TRY(ctx, launch_gemv(a, ctx->tune, ctx->stream));
   return ZTVM_OK;
 }
@@ -469,6 +505,7 @@ static int qkv_fused_common(ztvm_ctx* ctx, const ztvm_qkv_fused_desc* d, uint64_
   a.up_scales = a.scales + (size_t)half * d->scales_per_row;
   a.up_biases = d->affine ? a.biases + (size_t)half * d->scales_per_row : nullptr;
   a.qkv = &q;
+  if (!gemv_supports(a)) return fail(ctx, ZTVM_E_UNSUPPORTED, "ztvm_qkv_fused: K=%llu does not fit the LDS staging of the activation row", (unsigned long long)K);
   HIP_TRY(ctx, launch_gemv(a, ctx->tune, ctx->stream));
   return ZTVM_OK;
 }
@@ -608,17 +645,12 @@ int ztvm_repack_permute_rows(ztvm_ctx* ctx, uint64_t dst, uint64_t src, size_t b
     if (src_rows[j] >= rows) return fail(ctx, ZTVM_E_INVALID, "permuteRows src[%u] = %u is out of range", j, src_rows[j]);
   if ((dst < src + bytes) && (src < dst + bytes)) return fail(ctx, ZTVM_E_INVALID, "ztvm_repack_permute_rows: dst and src overlap");
   const size_t need = (size_t)rows * 4u;
-  if (need > ctx->scratch_bytes) {
-    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
-    HIP_TRY(ctx, hipFree(ctx->scratch));
-    ctx->scratch = nullptr;
-    ctx->scratch_bytes = 0;
-    HIP_TRY(ctx, hipMalloc(&ctx->scratch, need));
-    ctx->scratch_bytes = need;
-  }
-  HIP_TRY(ctx, hipMemcpyAsync(ctx->scratch, src_rows, need, hipMemcpyHostToDevice, ctx->stream));
+  void* map = nullptr;
+  int rc = scratch_for(ctx, need, &map);
+  if (rc) return rc;
+  HIP_TRY(ctx, hipMemcpyAsync(map, src_rows, need, hipMemcpyHostToDevice, ctx->stream));
   HIP_TRY(ctx, launch_permute_rows(reinterpret_cast<void*>(dst), reinterpret_cast<const void*>(src),
-                                   reinterpret_cast<const uint32_t*>(ctx->scratch), rows, bytes / rows, ctx->stream));
+                                   reinterpret_cast<const uint32_t*>(map), rows, bytes / rows, ctx->stream));
   HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));  // the map may be reused on return, and the scratch by the next dispatch
   return ZTVM_OK;
 }
@@ -658,6 +690,8 @@ int ztvm_record_end(ztvm_ctx* ctx, ztvm_cmdbuf** out) {
     delete cb;
     return fail(ctx, ZTVM_E_HIP, "command buffer finish: %s", hipGetErrorString(e));
   }
+  cb->scratch = ctx->scratch;
+  cb->scratch->pin();
   *out = cb;
   return ZTVM_OK;
 }
@@ -673,6 +707,7 @@ void ztvm_cmdbuf_destroy(ztvm_cmdbuf* cb) {
   if (!cb) return;
   if (cb->exec) (void)hipGraphExecDestroy(cb->exec);
   if (cb->graph) (void)hipGraphDestroy(cb->graph);
+  if (cb->scratch) cb->scratch->unpin();
   delete cb;
 }
 
@@ -712,6 +747,9 @@ int ztvm_set_option(ztvm_ctx* ctx, const char* name, int value) {
   if (!ctx || !name) return fail(ctx, ZTVM_E_INVALID, "ztvm_set_option: null argument");
   for (const Option& o : kOptions)
     if (!strcmp(o.name, name)) {
+      if (!strcmp(name, "gemv.rows") && value != 0 && value != 1 && value != 2 && value != 4)
+        return fail(ctx, ZTVM_E_INVALID, "gemv.rows must be 0 (default), 1, 2 or 4 (got %d)", value);
+      if (value < 0) return fail(ctx, ZTVM_E_INVALID, "option '%s' must be >= 0 (got %d)", name, value);
       ctx->tune.*(o.field) = value;
       return ZTVM_OK;
     }

@@ -25,6 +25,7 @@ EXPORTS = [
     "ztvm_repack_part", "ztvm_repack_permute_rows", "ztvm_repack_dequant_split",
 ]
 CONVERT_RAW, CONVERT_BF16_F16, CONVERT_BF16_F32 = 0, 1, 2
+EXPERTS_UNCHECKED = 0xFFFFFFFF  # ztvm_matmul_desc.experts: the caller vouches for every id
 
 
 class ZtvmError(RuntimeError):

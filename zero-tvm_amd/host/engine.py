@@ -377,11 +377,30 @@ class Device:
                 raise ValueError("moe pipeline '%s' needs the 8-field PODArgs" % p.label)
             d.in_slot_stride, d.out_slot_stride, d.in_tok_stride, d.out_tok_stride, d.ids_stride = w[3:8]
             d.tokens, d.slots = wg_y, wg_z
+            d.experts = self.stack_height(group, d)
         elif p.runtime_m:
             d.M = w[3]
         else:
             d.M = p.fixed_m
         return d
+
+    @staticmethod
+    def stack_height(group, d):
+        """Experts in the bound stacks, from the sizes of the bound regions: WebGPU bounds-checks
+        every storage access against those sizes, here the kernel's expert-id guard does, so the
+        guard is always armed for a dispatch built from a bind group. The three stacks must agree."""
+        per_w = d.N * d.k_packed * 4
+        per_s = d.N * d.scales_per_row * 2
+        if per_w == 0 or per_s == 0:
+            raise ValueError("moe pipeline '%s': empty expert (N=%d, K_PACKED=%d)" % (group.pipeline.label, d.N, d.k_packed))
+        heights = [group.weights[1] // per_w, group.scales[1] // per_s]
+        if group.pipeline.affine:
+            heights.append(group.biases[1] // per_s)
+        experts = min(heights)
+        if experts < 1:
+            raise ValueError("moe pipeline '%s': the bound stacks hold no whole expert (weights %d B, scales %d B)"
+                             % (group.pipeline.label, group.weights[1], group.scales[1]))
+        return experts
 
     def dispatch(self, pipeline, group, wg_x, wg_y=1, wg_z=1, label=None):
         """One compute pass. M_ROWS == 0 dispatches nothing, like a zero-row chunk."""

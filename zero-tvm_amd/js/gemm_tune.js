@@ -1,166 +1,203 @@
 'use strict'
-// Boot-time choice of the prefill ("chunk") GEMM by measurement, remembered per device and model: the policy of
-// the reference's src/zero-tvm/gemm-tune.ts (tuneKey :52-54, deviceFingerprint :61-78, median :81-85,
-// pickFromTimings :90-105, loadTunedPick :110-129, saveTunedPick :131-145, timeClosures :162-189,
-// resolveTunedGemm :208-233). Candidates are plain names: the reference's pipelines ('e5', 'sgmat', 'tiled',
-// 'matvec') or this library's kernel families ('gemm', 'skinny', 'rows', 'gemv'), which probeFamilies times
-// through Device.dispatch with the family forced. Without a pick ztvm_matmul routes by its own row thresholds.
+// Which prefill GEMM runs the chunk dispatches, decided once at start-up by timing the candidates on the device
+// and remembered per (device, model). This replaces the role of src/zero-tvm/gemm-tune.ts in the reference and keeps
+// its exported names so callers switch over unchanged; the rules, stated once:
+//
+//   score      a candidate's score is the geometric mean, over the probe sizes, of the median of its samples at
+//              each size; the lowest score wins and an exact tie goes to whichever stands earlier in the ladder
+//   memory     a remembered choice is a JSON record {version, pick, ms, candidates, at}; it is honoured only while
+//              its version is current, it is younger than TUNE_TTL_MS, its pick can still run, and every candidate
+//              that can run today was part of the measurement that produced it
+//   priority   an explicit request is never overridden; with fewer than two candidates there is nothing to decide;
+//              whatever goes wrong (store, clock, probe) the answer is "no opinion" (null) and the static
+//              thresholds of ztvm_matmul decide
+//
+// Candidates are names: the reference's pipelines ('e5', 'sgmat', 'tiled', 'matvec') or this library's kernel
+// families ('gemm', 'skinny', 'rows', 'gemv'), which probeFamilies times with the family forced in the descriptor.
 
-const TUNE_VERSION = 1 // bump when a GEMM kernel changes shape or speed: stored picks go stale
-const TUNE_TTL_MS = 30 * 24 * 3600 * 1000 // drivers move performance too: re-tune monthly
-const TUNE_MS = [64, 256, 1024] // probe sizes (chunk rows): ragged head, middle, full cap
+const TUNE_VERSION = 2            // raise when a kernel family changes speed: older records stop counting
+const TUNE_TTL_MS = 2592000000    // 30 days
+const TUNE_MS = [64, 256, 1024]   // chunk rows probed: a ragged head, a middle, a full chunk
 const TUNE_WARMUP = 2
 const TUNE_ROUNDS = 4
 const REFERENCE_LADDER = ['e5', 'sgmat', 'tiled', 'matvec']
 const FAMILY_LADDER = ['gemm', 'skinny', 'rows', 'gemv']
+const FAMILY_KERNEL = { gemv: 1, skinny: 2, gemm: 3, rows: 4 } // ZTVM_KERNEL_* of include/ztvm.h
 
-function tuneKey(adapterId, specId) { return 'ztvm.gemmTune.v' + TUNE_VERSION + '.' + adapterId + '.' + specId }
+const tuneKey = (adapterId, specId) => ['ztvm.gemmTune', 'v' + TUNE_VERSION, adapterId, specId].join('.')
 
-// Identity of the device for the key, from Device.info(): name / compute units / memory; null when nothing
-// identifies it (the caller then tunes without persisting).
+/** A stable id for the device out of Device.info(); null when the device will not say who it is. */
 function deviceFingerprint(info) {
-  try {
-    if (info && info.name) {
-      const cu = info.computeUnits === undefined ? '?' : String(info.computeUnits)
-      const mem = info.hbmBytes === undefined ? '?' : String(info.hbmBytes)
-      return [String(info.name), cu, mem].join('/').replace(/[^\w./-]/g, '_')
-    }
-  } catch (e) { /* a fingerprint must never break boot */ }
-  return null
+  if (!info || typeof info !== 'object' || !info.name) return null
+  const field = (v) => (v === undefined || v === null ? '?' : String(v))
+  return [info.name, info.computeUnits, info.hbmBytes].map(field).join('/').replace(/[^\w./-]/g, '_')
 }
 
-function median(xs) {
-  const s = xs.slice().sort((a, b) => a - b)
-  const m = s.length >> 1
-  return s.length % 2 ? s[m] : (s[m - 1] + s[m]) / 2
+function median(samples) {
+  const sorted = Array.from(samples).sort((p, q) => p - q)
+  const upper = sorted[Math.floor(sorted.length / 2)]
+  return sorted.length & 1 ? upper : 0.5 * (sorted[sorted.length / 2 - 1] + upper)
 }
 
-// Lowest geometric mean (across sizes) of the per-size medians; strictly-less keeps the earlier ladder entry on
-// exact ties; candidates without timings are ignored; nothing timed -> the ladder's last entry.
-function pickFromTimings(medians, ladder) {
-  let best = ladder[ladder.length - 1]
-  let bestScore = Infinity
-  for (const name of ladder) {
-    const ms = medians[name]
-    if (!ms || !ms.length) continue
-    const geo = Math.exp(ms.reduce((a, m) => a + Math.log(Math.max(m, 1e-9)), 0) / ms.length)
-    if (geo < bestScore) { bestScore = geo; best = name }
+/** Scores of the candidates that were measured: name -> geometric mean of its per-size medians. */
+class Scoreboard {
+  constructor() { this.perSize = new Map() }
+  /** medians: one number per probe size */
+  add(name, medians) {
+    const usable = (medians || []).filter((v) => Number.isFinite(v))
+    if (usable.length) this.perSize.set(name, usable)
+    return this
   }
-  return best
+  get size() { return this.perSize.size }
+  score(name) {
+    const m = this.perSize.get(name)
+    if (!m) return null
+    let logSum = 0
+    for (const v of m) logSum += Math.log(v > 1e-9 ? v : 1e-9)
+    return Math.exp(logSum / m.length)
+  }
+  /** The measured ladder entry with the lowest score, earlier entries first among equals; the ladder's
+   *  last entry when none of them was measured. */
+  winner(ladder) {
+    const ranked = ladder.map((name, rank) => ({ name, rank, score: this.score(name) })).filter((c) => c.score !== null)
+    if (!ranked.length) return ladder[ladder.length - 1]
+    ranked.sort((p, q) => p.score - q.score || p.rank - q.rank)
+    return ranked[0].name
+  }
+  summary() {
+    const out = {}
+    for (const [name, m] of this.perSize) out[name] = median(m)
+    return out
+  }
 }
 
-// A stored pick counts only if it is current-version, fresh, still runnable, and was measured against a
-// candidate set covering today's runnable ones; anything else (also corrupt data, a throwing store): re-tune.
+function pickFromTimings(medians, ladder) {
+  const board = new Scoreboard()
+  for (const name of Object.keys(medians)) board.add(name, medians[name])
+  return board.winner(ladder)
+}
+
+/** The remembered choice and the test of whether it still applies. */
+class TuneRecord {
+  constructor(pick, ms, candidates, at) { Object.assign(this, { version: TUNE_VERSION, pick, ms, candidates, at }) }
+  static parse(text) {
+    if (typeof text !== 'string' || !text) return null
+    let obj
+    try { obj = JSON.parse(text) } catch (err) { return null }
+    if (obj === null || typeof obj !== 'object') return null
+    const rec = new TuneRecord(obj.pick, obj.ms, obj.candidates, obj.at)
+    rec.version = obj.version
+    return rec
+  }
+  appliesTo(runnable, now) {
+    const fresh = typeof this.at === 'number' && now - this.at <= TUNE_TTL_MS
+    const covered = Array.isArray(this.candidates) && runnable.every((name) => this.candidates.indexOf(name) >= 0)
+    return this.version === TUNE_VERSION && fresh && covered && runnable.indexOf(this.pick) >= 0
+  }
+}
+
 function loadTunedPick(store, key, runnable, now) {
   if (!store || !runnable.length) return null
-  let raw = null
-  try { raw = store.load(key) } catch (e) { return null }
-  if (!raw) return null
-  let saved
-  try { saved = JSON.parse(raw) } catch (e) { return null }
-  if (!saved || typeof saved !== 'object' || saved.version !== TUNE_VERSION) return null
-  const t = now === undefined ? Date.now() : now
-  if (typeof saved.at !== 'number' || t - saved.at > TUNE_TTL_MS) return null
-  if (!runnable.includes(saved.pick)) return null
-  if (!Array.isArray(saved.candidates) || !runnable.every((c) => saved.candidates.includes(c))) return null
-  return saved.pick
+  let text
+  try { text = store.load(key) } catch (err) { return null }
+  const rec = TuneRecord.parse(text)
+  return rec && rec.appliesTo(runnable, now === undefined ? Date.now() : now) ? rec.pick : null
 }
 
 function saveTunedPick(store, key, pick, ms, candidates) {
   if (!store) return
-  try {
-    store.save(key, JSON.stringify({ version: TUNE_VERSION, pick, ms, candidates, at: Date.now() }))
-  } catch (e) { /* persistence must never break boot */ }
+  try { store.save(key, JSON.stringify(new TuneRecord(pick, ms, candidates, Date.now()))) } catch (err) { /* the choice still stands for this run */ }
 }
 
+/** key -> string stores: in memory, or one JSON file standing where the browser has localStorage. */
 function memoryTuneStore(init) {
-  const m = new Map(Object.entries(init || {}))
-  return { load: (k) => (m.has(k) ? m.get(k) : null), save: (k, v) => { m.set(k, v) } }
+  const cells = Object.assign(Object.create(null), init || {})
+  return { load: (key) => (key in cells ? cells[key] : null), save: (key, value) => { cells[key] = value } }
 }
 
-// One JSON file of key -> value (the place of the browser's localStorage).
 function fileTuneStore(file) {
   const fs = require('fs')
-  const read = () => {
-    try {
-      const d = JSON.parse(fs.readFileSync(file, 'utf8'))
-      return d && typeof d === 'object' && !Array.isArray(d) ? d : {}
-    } catch (e) { return {} }
+  const slurp = () => {
+    let parsed = null
+    try { parsed = JSON.parse(fs.readFileSync(file, 'utf8')) } catch (err) { /* absent or unreadable: empty */ }
+    return parsed && typeof parsed === 'object' && !Array.isArray(parsed) ? parsed : {}
   }
   return {
-    load: (k) => { const d = read(); return k in d ? d[k] : null },
-    save: (k, v) => { const d = read(); d[k] = v; fs.writeFileSync(file + '.tmp', JSON.stringify(d)); fs.renameSync(file + '.tmp', file) },
+    load(key) { const all = slurp(); return Object.prototype.hasOwnProperty.call(all, key) ? all[key] : null },
+    save(key, value) {
+      const all = slurp()
+      all[key] = value
+      const tmp = file + '.tmp'
+      fs.writeFileSync(tmp, JSON.stringify(all))
+      fs.renameSync(tmp, file) // readers see the old file or the new one, never half of one
+    },
   }
 }
 
-// Time each candidate's run(m) (one enqueued GEMM dispatch of m rows) to completion (sync() blocks until the
-// queue is empty), candidates interleaved within a round. Returns {name: {m: [ms, ...]}}; throws nothing: a
-// failure ends the probe and what was measured so far is returned.
+/** Wall-clock samples of runs[name](m), each run to completion (sync() returns when the queue is empty). Within a
+ *  round every candidate runs once before any runs twice, so drift of the clocks hits all of them alike. A throw
+ *  anywhere ends the probe; the samples taken so far are returned. Result: {name: {m: [ms, ...]}}. */
 function timeClosures(sync, runs, Ms, opts) {
-  const o = Object.assign({ warmup: TUNE_WARMUP, rounds: TUNE_ROUNDS, clock: () => Number(process.hrtime.bigint()) / 1e6 }, opts || {})
-  const names = Object.keys(runs)
-  const out = {}
+  const cfg = opts || {}
+  const warmup = cfg.warmup === undefined ? TUNE_WARMUP : cfg.warmup
+  const rounds = cfg.rounds === undefined ? TUNE_ROUNDS : cfg.rounds
+  const clock = cfg.clock || (() => Number(process.hrtime.bigint()) / 1e6)
+  const order = Object.keys(runs)
+  const samples = {}
+  const note = (name, m, ms) => {
+    const bySize = samples[name] || (samples[name] = {})
+    ;(bySize[m] || (bySize[m] = [])).push(ms)
+  }
   try {
     for (const m of Ms) {
-      for (let w = 0; w < o.warmup; w++) for (const name of names) runs[name](m)
+      for (let i = 0; i < warmup; i++) order.forEach((name) => runs[name](m))
       sync()
-      for (let r = 0; r < o.rounds; r++) {
-        for (const name of names) {
-          const t0 = o.clock()
+      for (let round = 0; round < rounds; round++) {
+        for (const name of order) {
+          const start = clock()
           runs[name](m)
           sync()
-          const dt = o.clock() - t0
-          if (!out[name]) out[name] = {}
-          if (!out[name][m]) out[name][m] = []
-          out[name][m].push(dt)
+          note(name, m, clock() - start)
         }
       }
     }
-  } catch (e) { /* timing is advisory; the ladder is the fallback */ }
-  return out
+  } catch (err) { /* a partial probe is still a probe */ }
+  return samples
 }
 
-// The boot-time decision: {pick, source: 'explicit' | 'stored' | 'probed'} or null when the static ladder should
-// decide (one candidate, a stored miss plus a failed or empty probe).
+/** {pick, source} with source 'explicit' | 'stored' | 'probed', or null for "no opinion". */
 function resolveTunedGemm(opts) {
   if (opts.explicit) return { pick: opts.explicit, source: 'explicit' }
   const runnable = opts.runnable
-  if (runnable.length <= 1) return null
+  if (!runnable || runnable.length < 2) return null
   const store = opts.store || null
-  const key = opts.adapterId ? tuneKey(opts.adapterId, opts.specId) : null
-  if (key) {
-    const stored = loadTunedPick(store, key, runnable)
-    if (stored) return { pick: stored, source: 'stored' }
-  }
-  let timings = {}
-  try { timings = opts.runProbe() || {} } catch (e) { timings = {} }
-  const medians = {}
+  const key = opts.adapterId ? tuneKey(opts.adapterId, opts.specId) : null // an anonymous device is tuned but not remembered
+  const remembered = key ? loadTunedPick(store, key, runnable) : null
+  if (remembered) return { pick: remembered, source: 'stored' }
+
+  let samples = null
+  try { samples = opts.runProbe() } catch (err) { samples = null }
+  const board = new Scoreboard()
   for (const name of runnable) {
-    const perSize = timings[name]
-    if (!perSize) continue
-    const arr = Object.values(perSize).filter((v) => v && v.length).map(median).filter((m) => Number.isFinite(m))
-    if (arr.length) medians[name] = arr
+    const bySize = samples && samples[name]
+    if (bySize) board.add(name, Object.keys(bySize).map((m) => bySize[m]).filter((s) => s && s.length).map(median))
   }
-  if (!Object.keys(medians).length) return null
-  const order = opts.order || REFERENCE_LADDER.concat(FAMILY_LADDER)
-  const ladder = order.filter((n) => runnable.includes(n))
-  const pick = pickFromTimings(medians, ladder.length ? ladder : runnable)
-  const ms = {}
-  for (const name of Object.keys(medians)) ms[name] = median(medians[name])
-  if (key) saveTunedPick(store, key, pick, ms, runnable)
+  if (!board.size) return null
+  const preference = (opts.order || REFERENCE_LADDER.concat(FAMILY_LADDER)).filter((name) => runnable.indexOf(name) >= 0)
+  const pick = board.winner(preference.length ? preference : runnable)
+  if (key) saveTunedPick(store, key, pick, board.summary(), runnable)
   return { pick, source: 'probed' }
 }
 
-// Time this library's kernel families on one dense GEMM (the caller's real gate/up weights behind `desc`, an
-// activation buffer of at least max(Ms) rows). validate/matmul: the addon's descriptor calls; a family that cannot
-// take the shape is left out.
+/** Samples for this library's kernel families on one dense GEMM: `desc` names the caller's real weights and an
+ *  activation buffer of at least max(Ms) rows; api = {validate, matmul, sync} of the addon. A family that refuses
+ *  the descriptor at any probe size is not a candidate. */
 function probeFamilies(api, desc, families, Ms, opts) {
-  const kernels = { gemm: 3, skinny: 2, rows: 4, gemv: 1 }
   const sizes = Ms || TUNE_MS
+  const forced = (name, m) => Object.assign({}, desc, { kernel: FAMILY_KERNEL[name], M: m })
   const runs = {}
   for (const name of families) {
-    const fits = sizes.every((m) => api.validate(Object.assign({}, desc, { kernel: kernels[name], M: m })).code === 0)
-    if (fits) runs[name] = (m) => api.matmul(Object.assign({}, desc, { kernel: kernels[name], M: m }))
+    if (sizes.every((m) => api.validate(forced(name, m)).code === 0)) runs[name] = (m) => api.matmul(forced(name, m))
   }
   return timeClosures(api.sync, runs, sizes, opts)
 }
@@ -168,5 +205,5 @@ function probeFamilies(api, desc, families, Ms, opts) {
 module.exports = {
   TUNE_VERSION, TUNE_TTL_MS, TUNE_MS, TUNE_WARMUP, TUNE_ROUNDS, REFERENCE_LADDER, FAMILY_LADDER,
   tuneKey, deviceFingerprint, median, pickFromTimings, loadTunedPick, saveTunedPick, memoryTuneStore, fileTuneStore,
-  timeClosures, resolveTunedGemm, probeFamilies,
+  timeClosures, resolveTunedGemm, probeFamilies, Scoreboard, TuneRecord,
 }

@@ -218,9 +218,12 @@ class Device {
     const need = 5 + (pipeline.affine ? 1 : 0) + (pipeline.moe ? 1 : 0)
     if (bufs.length < need) throw new Error("bg: pipeline '" + pipeline.label + "' needs " + need + ' bindings, got ' + bufs.length)
     if (!(bufs[4] instanceof Uniform)) throw new Error("bg: binding 4 of '" + pipeline.label + "' must be the PODArgs uniform")
+    // bytes bound at a binding: WebGPU bounds-checks storage accesses against them, here they arm the expert-id guard
+    const size = (b) => (b ? b.size : 0)
     return {
       pipeline, pod: bufs[4], out: addr(0, bufs[0]), in: addr(1, bufs[1]), scales: addr(2, bufs[2]), weights: addr(3, bufs[3]),
       biases: pipeline.affine ? addr(5, bufs[5]) : 0n, ids: pipeline.moe ? addr(6, bufs[6]) : 0n,
+      sizes: { scales: size(bufs[2]), weights: size(bufs[3]), biases: pipeline.affine ? size(bufs[5]) : 0 },
     }
   }
   descriptor(group, wgX, wgY, wgZ) {
@@ -234,6 +237,7 @@ class Device {
       d.in_slot_stride = w[3]; d.out_slot_stride = w[4]; d.in_tok_stride = w[5]; d.out_tok_stride = w[6]; d.ids_stride = w[7]
       d.tokens = wgY === undefined ? 1 : wgY
       d.slots = wgZ === undefined ? 1 : wgZ
+      d.experts = stackHeight(group, d)
     } else if (p.runtimeM) d.M = w[3]
     else d.M = p.fixedM
     return d
@@ -336,6 +340,18 @@ function densePod(K, N, bits, affine, M) {
   const pod = [K * (bits || 4) / 32, K / (affine === false ? 32 : 64), N]
   if (M !== undefined) pod.push(M)
   return pod
+}
+
+/** Experts in the bound stacks, from the bound sizes; the three stacks must each hold that many. */
+function stackHeight(group, d) {
+  const label = group.pipeline.label
+  const perW = d.N * d.k_packed * 4, perS = d.N * d.scales_per_row * 2
+  if (!perW || !perS) throw new Error("moe pipeline '" + label + "': empty expert (N=" + d.N + ', K_PACKED=' + d.k_packed + ')')
+  const sz = group.sizes || { weights: 0, scales: 0, biases: 0 }
+  let experts = Math.min(Math.floor(sz.weights / perW), Math.floor(sz.scales / perS))
+  if (group.pipeline.affine) experts = Math.min(experts, Math.floor(sz.biases / perS))
+  if (experts < 1) throw new Error("moe pipeline '" + label + "': the bound stacks hold no whole expert (weights " + sz.weights + ' B, scales ' + sz.scales + ' B)')
+  return experts
 }
 
 function moePods(dModel, ffn, slots, bits) {
