@@ -35,6 +35,9 @@ extern "C" {
 /* ztvm_matmul_desc.experts: the caller vouches for every id in ids[] */
 #define ZTVM_EXPERTS_UNCHECKED 0xFFFFFFFFu
 
+/* Bytes of device memory ztvm_matmul_static may use as scratch (held per GPU until the process ends). */
+#define ZTVM_STATIC_SCRATCH_BYTES (16u << 20)
+
 
 #if defined(__GNUC__)
 #define ZTVM_API __attribute__((visibility("default")))
@@ -170,6 +173,18 @@ ZTVM_API int ztvm_matmul(ztvm_ctx* ctx, const ztvm_matmul_desc* desc);
  * buffer that a live command buffer may reference: it is kept until the last such command buffer
  * is destroyed, so a command buffer recorded earlier stays valid to submit after any later
  * dispatch. Destroying the context ends the life of its command buffers. */
+
+/* ztvm_matmul for callers that cannot allocate device memory: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc. It has no counterpart in the reference. Same
+ * descriptor, same kernels and bit-identical results, but the scratch of the rows, skinny and
+ * tile-GEMM families is a fixed array of ZTVM_STATIC_SCRATCH_BYTES that lives in the library's
+ * device image (one copy per GPU, held until the process ends), so this call never calls hipMalloc
+ * or hipFree, whatever the shape. A dispatch that needs more scratch than that is refused with
+ * ZTVM_E_UNSUPPORTED and a message that says how much (ztvm_matmul takes any size). Nothing in the
+ * array has to start at zero: every kernel writes what it later reads. All calls on one GPU share
+ * the array, from every context and thread: two ztvm_matmul_static dispatches that overlap on one
+ * GPU (different contexts or streams) race on it; dispatches on one context are ordered and safe. */
+ZTVM_API int ztvm_matmul_static(ztvm_ctx* ctx, const ztvm_matmul_desc* desc);
 
 /* Gate + up + SiLU in one pass over the activations: out[n] = up[n] * silu(gate[n]) with
  * gate = W_gate x (the descriptor's weights / scales / biases) and up = W_up x (the three

@@ -32,6 +32,32 @@ struct DeviceAlloc {
   }
 };
 using DevicePool = ScratchPool<DeviceAlloc>;
+
+// Scratch of ztvm_matmul_static: device memory that exists from the moment the library's code object
+// is loaded, so the entry point never allocates. Every GPU the library runs on holds its own copy at
+// its own address; host code must only ever use the per-device address that hipGetSymbolAddress
+// returned (the array's name is not a device address on the host side).
+static __device__ __align__(256) __attribute__((used)) unsigned char static_scratch[ZTVM_STATIC_SCRATCH_BYTES];
+constexpr int kMaxDevices = 64;
+std::mutex g_static_mu;
+void* g_static_ptr[kMaxDevices] = {};
+
+// Address of `device`'s copy of the array, looked up once per device with that device current.
+hipError_t static_scratch_of(int device, void** out) {
+  if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(g_static_mu);
+  if (!g_static_ptr[device]) {
+    hipError_t e = hipSetDevice(device);
+    if (e != hipSuccess) return e;
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(static_scratch));
+    if (e != hipSuccess) return e;
+    if (!p) return hipErrorInvalidSymbol;
+    g_static_ptr[device] = p;
+  }
+  *out = g_static_ptr[device];
+  return hipSuccess;
+}
 }  // namespace
 
 struct ztvm_ctx {
@@ -43,6 +69,7 @@ struct ztvm_ctx {
   // reordered activations, split-k partial sums). Shared with the command buffers recorded on this
   // context, which keep its addresses alive (scratch_pool.h).
   std::shared_ptr<DevicePool> scratch;
+  void* static_scratch = nullptr;  // this device's copy of the file-scope array above
   std::string err;
   hipDeviceProp_t prop;
 };
@@ -250,6 +277,14 @@ int ztvm_create(int device, ztvm_ctx** out) {
   }
   HIP_TRY(nullptr, hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
   c->tune.num_cus = c->prop.multiProcessorCount > 0 ? c->prop.multiProcessorCount : 256;
+  {
+    hipError_t e = static_scratch_of(device, &c->static_scratch);
+    if (e != hipSuccess) {
+      (void)hipStreamDestroy(c->stream);
+      delete c;
+      return fail(nullptr, ZTVM_E_HIP, "ztvm_create: address of the static scratch array: %s", hipGetErrorString(e));
+    }
+  }
   c->scratch = std::make_shared<DevicePool>(DeviceAlloc{device});
   if (!c->scratch->reserve(4u << 20)) {
     (void)hipStreamDestroy(c->stream);
@@ -357,7 +392,8 @@ int ztvm_matmul_resolve(const ztvm_matmul_desc* desc) {
   return rc;
 }
 
-int ztvm_matmul(ztvm_ctx* ctx, const ztvm_matmul_desc* desc) {
+// use_static: the scratch is this device's copy of the file-scope array, nothing is allocated
+static int matmul_impl(ztvm_ctx* ctx, const ztvm_matmul_desc* desc, bool use_static) {
   if (!ctx) return fail(nullptr, ZTVM_E_INVALID, "null context");
   char why[256];
   int rc = validate(desc, why, sizeof why, true);
@@ -371,8 +407,15 @@ int ztvm_matmul(ztvm_ctx* ctx, const ztvm_matmul_desc* desc) {
     case ZTVM_KERNEL_GEMM: {
       const size_t need = fam == ZTVM_KERNEL_GEMM ? gemm_scratch_bytes(a) : (fam == ZTVM_KERNEL_ROWS ? rows_scratch_bytes(a) : skinny_scratch_bytes(a, ctx->tune));
       void* scratch = nullptr;
-      rc = scratch_for(ctx, need, &scratch);
-      if (rc) return rc;
+      if (use_static) {
+        if (need > (size_t)ZTVM_STATIC_SCRATCH_BYTES)
+          return fail(ctx, ZTVM_E_UNSUPPORTED, "ztvm_matmul_static: this dispatch needs %zu bytes of scratch, the static buffer holds %zu (M=%u N=%u K=%u); use ztvm_matmul",
+                      need, (size_t)ZTVM_STATIC_SCRATCH_BYTES, a.M, a.N, a.K);
+        scratch = ctx->static_scratch;
+      } else {
+        rc = scratch_for(ctx, need, &scratch);
+        if (rc) return rc;
+      }
       if (fam == ZTVM_KERNEL_GEMM) HIP_TRY(ctx, launch_gemm(a, ctx->tune, scratch, ctx->stream));
       else if (fam == ZTVM_KERNEL_ROWS) HIP_TRY(ctx, launch_rows(a, ctx->tune, scratch, ctx->stream));
       else HIP_TRY(ctx, launch_skinny(a, ctx->tune, scratch, ctx->stream));
@@ -393,6 +436,10 @@ int ztvm_matmul(ztvm_ctx* ctx, const ztvm_matmul_desc* desc) {
   }
   return ZTVM_OK;
 }
+
+int ztvm_matmul(ztvm_ctx* ctx, const ztvm_matmul_desc* desc) { return matmul_impl(ctx, desc, false); }
+
+int ztvm_matmul_static(ztvm_ctx* ctx, const ztvm_matmul_desc* desc) { return matmul_impl(ctx, desc, true); }
 
 int ztvm_ffn_gated(ztvm_ctx* ctx, const ztvm_matmul_desc* desc, uint64_t up_weights, uint64_t up_scales, uint64_t up_biases) {
   if (!ctx) return fail(nullptr, ZTVM_E_INVALID, "null context");

@@ -16,7 +16,7 @@ E_INVALID, E_HIP, E_UNSUPPORTED, E_NODEVICE = -1, -2, -3, -4
 EXPORTS = [
     "ztvm_abi_version", "ztvm_last_error", "ztvm_create", "ztvm_destroy", "ztvm_device_info",
     "ztvm_alloc", "ztvm_free", "ztvm_upload", "ztvm_download", "ztvm_fill", "ztvm_copy", "ztvm_sync",
-    "ztvm_matmul_validate", "ztvm_matmul_resolve", "ztvm_matmul", "ztvm_ffn_gated", "ztvm_ffn_gated_prologue", "ztvm_qkv_fused", "ztvm_qkv_fused_scratch",
+    "ztvm_matmul_validate", "ztvm_matmul_resolve", "ztvm_matmul", "ztvm_matmul_static", "ztvm_ffn_gated", "ztvm_ffn_gated_prologue", "ztvm_qkv_fused", "ztvm_qkv_fused_scratch",
     "ztvm_kv_quantize_int8", "ztvm_dequant",
     "ztvm_record_begin", "ztvm_record_end", "ztvm_submit", "ztvm_cmdbuf_destroy",
     "ztvm_event_create", "ztvm_event_destroy", "ztvm_event_record", "ztvm_event_elapsed_ms",
@@ -87,6 +87,7 @@ def load():
     L.ztvm_matmul_validate.argtypes = [C.POINTER(MatmulDesc), C.c_char_p, C.c_size_t]
     L.ztvm_matmul_resolve.argtypes = [C.POINTER(MatmulDesc)]
     L.ztvm_matmul.argtypes = [vp, C.POINTER(MatmulDesc)]
+    L.ztvm_matmul_static.argtypes = [vp, C.POINTER(MatmulDesc)]
     L.ztvm_dequant.argtypes = [vp, C.POINTER(MatmulDesc)]
     L.ztvm_record_begin.argtypes = [vp]
     L.ztvm_record_end.argtypes = [vp, C.POINTER(vp)]
@@ -194,6 +195,10 @@ class Context:
 
     def matmul(self, desc):
         self._chk(self._L.ztvm_matmul(self._h, C.byref(desc)))
+
+    def matmul_static(self, desc):
+        """ztvm_matmul on the library's fixed scratch array: never allocates device memory."""
+        self._chk(self._L.ztvm_matmul_static(self._h, C.byref(desc)))
 
     def ffn_gated(self, desc, up_weights, up_scales, up_biases=0):
         self._chk(self._L.ztvm_ffn_gated(self._h, C.byref(desc), up_weights, up_scales, up_biases))
