@@ -48,6 +48,8 @@ struct Tune {
   int gemv_wg_per_cu = 0;   // workgroups resident per CU for the streaming GEMV
   int gemv_rows = 0;        // rows per wave step (1, 2 or 4)
   int gemv_waves = 0;       // waves per workgroup (4..8)
+  int gemv_ring = 0;        // passes in flight per wave of the streaming kernel (0: two; 1, 3)
+  int gemv_stream = 0;      // 0: dense single rows go to the register-resident streaming kernel where it applies; 1: never
   int skinny_ksplit = 0;     // workgroups sharing the k range of one skinny tile (0: chosen from M, N, K)
   int rows_wg_per_cu = 0;    // the row-group GEMV: workgroups per CU and waves per workgroup (0: chosen from the LDS it stages)
   int rows_waves = 0;
@@ -57,6 +59,9 @@ struct Tune {
 
 hipError_t launch_gemv(const MatmulArgs& a, const Tune& t, hipStream_t s);
 bool gemv_supports(const MatmulArgs& a);  // the activation row fits the LDS staging
+// the dense single-row streaming kernel (gemv_stream.hip)
+bool gemv_stream_supports(const MatmulArgs& a, const Tune& t);
+hipError_t launch_gemv_stream(const MatmulArgs& a, const Tune& t, hipStream_t s);
 hipError_t launch_skinny(const MatmulArgs& a, const Tune& t, void* scratch, hipStream_t s);
 size_t skinny_scratch_bytes(const MatmulArgs& a, const Tune& t);
 hipError_t launch_gemm(const MatmulArgs& a, const Tune& t, void* scratch, hipStream_t s);

@@ -245,6 +245,8 @@ const Option kOptions[] = {
     {"gemv.wg_per_cu", &Tune::gemv_wg_per_cu},
     {"gemv.rows", &Tune::gemv_rows},
     {"gemv.waves", &Tune::gemv_waves},
+    {"gemv.stream", &Tune::gemv_stream},
+    {"gemv.ring", &Tune::gemv_ring},
     {"skinny.ksplit", &Tune::skinny_ksplit},
     {"rows.wg_per_cu", &Tune::rows_wg_per_cu},
     {"rows.waves", &Tune::rows_waves},
@@ -430,7 +432,8 @@ static int matmul_impl(ztvm_ctx* ctx, const ztvm_matmul_desc* desc, bool use_sta
         r.in = a.in + (size_t)m * a.K;
         r.out = reinterpret_cast<char*>(a.out) + (size_t)m * a.N * out_elt;
         r.M = 1;
-        HIP_TRY(ctx, launch_gemv(r, ctx->tune, ctx->stream));
+        if (ctx->tune.gemv_stream == 0 && gemv_stream_supports(r, ctx->tune)) HIP_TRY(ctx, launch_gemv_stream(r, ctx->tune, ctx->stream));
+        else HIP_TRY(ctx, launch_gemv(r, ctx->tune, ctx->stream));
       }
     }
   }
@@ -796,6 +799,10 @@ int ztvm_set_option(ztvm_ctx* ctx, const char* name, int value) {
     if (!strcmp(o.name, name)) {
       if (!strcmp(name, "gemv.rows") && value != 0 && value != 1 && value != 2 && value != 4)
         return fail(ctx, ZTVM_E_INVALID, "gemv.rows must be 0 (default), 1, 2 or 4 (got %d)", value);
+      if (!strcmp(name, "gemv.ring") && (value < 0 || value > 3))
+        return fail(ctx, ZTVM_E_INVALID, "gemv.ring must be 0 (default), 1, 2 or 3 (got %d)", value);
+      if (!strcmp(name, "num_cus") && (value < 1 || value > 4096))
+        return fail(ctx, ZTVM_E_INVALID, "num_cus must be 1..4096 (got %d)", value);
       if (value < 0) return fail(ctx, ZTVM_E_INVALID, "option '%s' must be >= 0 (got %d)", name, value);
       ctx->tune.*(o.field) = value;
       return ZTVM_OK;
