@@ -7,6 +7,12 @@ One step = the three GEMVs on one weight set; steps rotate over distinct
 weight sets whose total exceeds the 256 MB last-level cache, so every step
 streams its weights from HBM. Inputs are resident in HBM before timing.
 
+Timing discipline (the reference's, scripts/kernel-ab-ours.mjs:75-99): outputs are validated against the
+oracle before anything is timed; every memory-bound row rotates over more than 256 MB of distinct
+operands (`rotation_MB` in the row); the headline is the median of ROUNDS timed replays of the recorded
+steps, one replay in flight at a time, with min and max beside it; a plain streaming read of the same
+byte count is timed the same way in the same run (`extra.hbm_read_probe_*`); clocks are recorded.
+
 Prints ONE JSON line: value = algorithmic weight GB/s over the timed steps,
 plus `roofline` (HBM) and `cpu_baseline` (the CPU oracle on the host cores).
 """
@@ -14,6 +20,7 @@ import argparse
 import importlib
 import json
 import os
+import subprocess
 import sys
 import time
 
@@ -27,6 +34,8 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 # `bench.py --pmc` (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from a 256 MiB copy);
 # summary in profiles/gemv_int4_configs1_hbm_traffic.md
 GEMV_TRAFFIC_BYTES_PER_LAUNCH = 26.96e6
+ROTATION_FLOOR_BYTES = 300e6   # distinct operand bytes a memory-bound row rotates over: past the 256 MB last-level cache
+ROUNDS = 5                     # timed replays of the headline; the median is reported
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense f16 MFMA, published
 
 GEMV_SHAPES = [("ffn_gate_or_up", 4096, 14336), ("ffn_down", 14336, 4096), ("qkv_fused", 4096, 6144)]
@@ -57,8 +66,9 @@ def _put(ctx, arr):
     return addr
 
 
-def timed_graph(ctx, launches, reps=1, warm=1):
+def timed_graph(ctx, launches, reps=1, warm=1, rounds=False):
     """Record `launches` (callables) into one command buffer, replay `warm` times untimed, then time `reps` replays.
+    Returns the mean milliseconds per replay, or with rounds=True the sorted list of the replays' times.
     Compute-bound rows pass warm > 1: after an idle stretch (the oracle check before a row is one) the clock takes
     tens of milliseconds of load to come back up (the M=512 GEMM: 88 us cold, 76 after a few ms, 72 sustained)."""
     ctx.record_begin()
@@ -70,16 +80,47 @@ def timed_graph(ctx, launches, reps=1, warm=1):
         ctx.submit(cb)
         ctx.sync()
     e0, e1 = ctx.event(), ctx.event()
-    ms = 0.0
+    times = []
     for _ in range(reps):
         ctx.event_record(e0)
         ctx.submit(cb)
         ctx.event_record(e1)
-        ms += ctx.elapsed_ms(e0, e1)
+        times.append(ctx.elapsed_ms(e0, e1))   # waits for the replay: one in flight at a time
     ctx.event_destroy(e0)
     ctx.event_destroy(e1)
     ctx.cmdbuf_destroy(cb)
-    return ms / reps
+    return sorted(times) if rounds else sum(times) / reps
+
+
+def n_sets(bytes_per_set):
+    """How many distinct operand sets a row rotates over to stay past the last-level cache."""
+    return int(ROTATION_FLOOR_BYTES // bytes_per_set) + 1
+
+
+def clocks():
+    """Clock and power state as rocm-smi reports it, for the record (empty if the tool is not there)."""
+    try:
+        out = subprocess.run(["rocm-smi", "--showclocks", "--showperflevel", "--showpower", "--json"], capture_output=True,
+                             text=True, timeout=20).stdout
+        card = next(iter(json.loads(out).values()))
+        keep = {}
+        for k, v in card.items():
+            kl = k.lower()
+            if any(t in kl for t in ("sclk", "mclk", "fclk", "performance level", "power")):
+                keep[k] = v
+        return keep
+    except Exception:
+        return {}
+
+
+def error_metrics(y, ref):
+    """The three denominators the reference's own checks use, side by side: |ref| + 1e-3
+    (tests/kernels/run.mjs:153), max |ref| (scripts/real-weights.mjs:72-73), max(1e-2, |ref|)
+    (scripts/gemm-bench.mjs:516), and the contract's |ref| + 1e-2."""
+    d = np.abs(np.asarray(y, np.float64) - ref)
+    a = np.abs(ref)
+    return {"ref_plus_1e-3": float(np.max(d / (a + 1e-3))), "max_abs_ref": float(np.max(d) / np.max(a)),
+            "max_1e-2_ref": float(np.max(d / np.maximum(a, 1e-2))), "ref_plus_1e-2": float(np.max(d / (a + 1e-2)))}
 
 
 def verify(ctx, oracle, capi, desc, host, bits, K, N, M, f16w=False):
@@ -181,26 +222,35 @@ def main():
         return
 
     # ---- headline: rotating weight sets, three GEMVs per step ------------------
-    sets = []
-    for r in range(args.sets):
-        per_shape = []
-        for i, (_, K, N) in enumerate(GEMV_SHAPES):
+    # per shape enough distinct sets to rotate past the last-level cache on its own (the small QKV shape needs
+    # twenty), so the per-shape rows below are HBM measurements too; step r takes set r % n of every shape
+    shape_sets, shape_hosts, shape_bytes = [], [], []
+    for i, (_, K, N) in enumerate(GEMV_SHAPES):
+        wb = synth.weight_bytes(N, K)
+        per_set, first_host = [], None
+        for r in range(max(args.sets, n_sets(wb))):
             bufs, host = upload_set(ctx, synth, K, N, 4, salt=10 * r + i)
             desc = make_desc(capi, 4, K, N, 1, bufs)
             if r == 0:
                 verify(ctx, oracle, capi, desc, host, 4, K, N, 1)
-            per_shape.append(desc)
-        sets.append(per_shape)
-    step_bytes = sum(synth.weight_bytes(N, K) for _, K, N in GEMV_SHAPES)
+                first_host = host
+            per_set.append(desc)
+        shape_sets.append(per_set)
+        shape_hosts.append(first_host)
+        shape_bytes.append(wb)
+    step_bytes = sum(shape_bytes)
+    rotation_bytes = sum(len(ss) * wb for ss, wb in zip(shape_sets, shape_bytes))
+    sets = [[ss[r % len(ss)] for ss in shape_sets] for r in range(max(len(ss) for ss in shape_sets))]  # sets[r][shape]
 
-    def step(i):
-        for desc in sets[i % args.sets]:
+    def step(i, table=None):
+        for desc in (table or sets)[i % len(sets)]:
             ctx.matmul(desc)
 
     for i in range(args.warmup):
         step(i)
     ctx.sync()
-    ms_total = timed_graph(ctx, [lambda i=i: step(i) for i in range(args.steps)])
+    rounds = timed_graph(ctx, [lambda i=i: step(i) for i in range(args.steps)], reps=ROUNDS, rounds=True)
+    ms_total = rounds[len(rounds) // 2]
     ms_per_step = ms_total / args.steps
     gbs = step_bytes / (ms_per_step * 1e-3) / 1e9
     launches = 3 * args.steps
@@ -212,44 +262,94 @@ def main():
         "ms_per_step": round(ms_per_step, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int4 weights (u32-packed), f16 activations, f32 accumulate", "data": "synthetic",
         "config": {"workload": "configs[1]: int4 affine g64 decode GEMV, M=1, (4096->14336)+(14336->4096)+(4096->6144) "
-                               "per step, %d rotating weight sets" % args.sets,
-                   "device": info["name"], "compute_units": info["compute_units"]},
+                               "per step, rotating over %.0f MB of distinct weights" % (rotation_bytes / 1e6),
+                   "device": info["name"], "compute_units": info["compute_units"], "rotation_MB": round(rotation_bytes / 1e6, 1),
+                   "timing": "median of %d replays of %d recorded steps, one replay in flight at a time" % (ROUNDS, args.steps),
+                   "ms_per_step_min": round(rounds[0] / args.steps, 6), "ms_per_step_max": round(rounds[-1] / args.steps, 6),
+                   "clocks": clocks()},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": GEMV_TRAFFIC_BYTES_PER_LAUNCH,
-                     "kernel": "ztvm::gemv_kernel<4,true,64,*>", "bytes_per_launch": step_bytes / 3.0,
+                     "kernel": "ztvm::gemv_stream_kernel<4,true,2,*,*>", "bytes_per_launch": step_bytes / 3.0,
                      "avg_launch_us": round(avg_launch_us, 3), "launches": launches},
     }
 
     if not args.no_extra:
         extra = {}
-        # per shape, each alone over its rotating sets
+        sink = ctx.alloc(64)
+        # per shape, each alone over its own rotating sets, with a plain streaming read of the same bytes beside it
+        # (the packed words of the same sets read by a kernel that does nothing else): the empirical ceiling
         for i, (name, K, N) in enumerate(GEMV_SHAPES):
-            reps = 40
-            ms = timed_graph(ctx, [lambda d=sets[j % args.sets][i]: ctx.matmul(d) for j in range(reps * args.sets)]) / (reps * args.sets)
-            wb = synth.weight_bytes(N, K)
+            ss, wb = shape_sets[i], shape_bytes[i]
+            reps = max(2, 160 // len(ss))
+            n = reps * len(ss)
+            ms = timed_graph(ctx, [lambda d=ss[j % len(ss)]: ctx.matmul(d) for j in range(n)], reps=ROUNDS, rounds=True)[ROUNDS // 2] / n
+            pb = N * (K // 8) * 4
+            ms_r = timed_graph(ctx, [lambda d=ss[j % len(ss)]: ctx.read_probe(d.weights, pb, sink) for j in range(n)], reps=ROUNDS,
+                               rounds=True)[ROUNDS // 2] / n
             extra["gemv_%s_K%d_N%d" % (name, K, N)] = {"us": round(ms * 1e3, 3), "GB/s": round(wb / ms / 1e6, 1),
-                                                       "hbm_frac": round(wb / ms / 1e6 / HBM_PEAK_GBS, 4)}
+                                                       "hbm_frac": round(wb / ms / 1e6 / HBM_PEAK_GBS, 4),
+                                                       "rotation_MB": round(len(ss) * wb / 1e6, 1)}
+            extra["hbm_read_probe_%.0fMB_%s" % (pb / 1e6, name)] = {"us": round(ms_r * 1e3, 3), "GB/s": round(pb / ms_r / 1e6, 1),
+                                                                   "hbm_frac": round(pb / ms_r / 1e6 / HBM_PEAK_GBS, 4),
+                                                                   "bytes": pb, "rotation_MB": round(len(ss) * pb / 1e6, 1)}
+        # bias regime B (MLX-like centred biases, b = -7.5 s (1 +- 0.1): every weight sits near zero and the two terms
+        # of s*dot + b*sum(x) cancel): same weights and scales, other biases; validated, then the same step timed.
+        # The errors of both regimes under the reference's three denominators are reported side by side.
+        errs = {}
+        setsB = []
+        for r in range(len(sets)):
+            rowB = []
+            for i, (_, K, N) in enumerate(GEMV_SHAPES):
+                d = sets[r][i]
+                if r < len(shape_sets[i]):
+                    sc_host = synth.scales(N, K, salt=10 * r + i)
+                    bB = synth.biases(N, K, sc_host, "B", salt=10 * r + i)
+                    dB = capi.MatmulDesc(bits=4, affine=1, M=1, N=N, k_packed=K // 8, scales_per_row=K // 64, out=d.out, in_=d.in_,
+                                         scales=d.scales, weights=d.weights, biases=_put(ctx, bB))
+                    if r == 0:
+                        x0, w0, s0, bA = shape_hosts[i]
+                        for regime, dd, bb in (("A", d, bA), ("B", dB, bB)):
+                            ctx.matmul(dd)
+                            y = ctx.download(dd.out, N * 2, np.float16).astype(np.float64)
+                            ref = oracle.gemm(oracle.MODE_FORMULA_F32, 4, True, 1, N, K, x0, w0, s0, bb, threads=oracle.max_threads())[0]
+                            m = error_metrics(y, ref)
+                            if m["ref_plus_1e-2"] >= 1e-2:
+                                raise SystemExit("bench: regime %s output check failed (K=%d N=%d): %r" % (regime, K, N, m))
+                            errs["regime%s_K%d_N%d" % (regime, K, N)] = {k: float("%.3g" % v) for k, v in m.items()}
+                    rowB.append(dB)
+                else:
+                    rowB.append(setsB[r % len(shape_sets[i])][i])
+            setsB.append(rowB)
+        msB = timed_graph(ctx, [lambda i=i: step(i, setsB) for i in range(args.steps)], reps=ROUNDS, rounds=True)[ROUNDS // 2] / args.steps
+        extra["gemv_step_bias_regime_B"] = {"ms_per_step": round(msB, 6), "GB/s": round(step_bytes / msB / 1e6, 1),
+                                            "hbm_frac": round(step_bytes / msB / 1e6 / HBM_PEAK_GBS, 4),
+                                            "rotation_MB": round(rotation_bytes / 1e6, 1)}
+        extra["gemv_max_rel_err_vs_fp32_accumulated_reference"] = errs
         # prefill GEMM (configs[2]): K=4096, N=14336, M in {128, 512, 2048}
         gsets = []
-        for r in range(3):
+        g_wb = synth.weight_bytes(14336, 4096)
+        for r in range(n_sets(g_wb)):
             bufs, host = upload_set(ctx, synth, 4096, 14336, 4, salt=100 + r, M=2048)
             gsets.append((bufs, host))
+        ng = len(gsets)
         for M in (128, 512, 2048):
             descs = [make_desc(capi, 4, 4096, 14336, M, b, kernel=capi.KERNEL_GEMM) for b, _ in gsets]
             verify(ctx, oracle, capi, descs[0], gsets[0][1], 4, 4096, 14336, M)
-            reps = 12 if M <= 512 else 4
-            ms = timed_graph(ctx, [lambda d=descs[j % 3]: ctx.matmul(d) for j in range(reps * 3)], reps=6, warm=6) / (reps * 3)
+            reps = 4 if M <= 512 else 1
+            ms = timed_graph(ctx, [lambda d=descs[j % ng]: ctx.matmul(d) for j in range(reps * ng)], reps=6, warm=6) / (reps * ng)
             tf = 2.0 * M * 4096 * 14336 / ms / 1e9
             extra["gemm_M%d_K4096_N14336" % M] = {"us": round(ms * 1e3, 2), "TFLOP/s": round(tf, 1),
-                                                  "mfma_f16_frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
+                                                  "mfma_f16_frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
+                                                  "rotation_MB": round(ng * (g_wb + M * 4096 * 2) / 1e6, 1)}
         # int3 decode GEMV (configs[4], M=1)
-        i3 = [upload_set(ctx, synth, 4096, 14336, 3, salt=200 + r) for r in range(8)]
+        wb = synth.weight_bytes(14336, 4096, bits=3)
+        n3 = n_sets(wb)
+        i3 = [upload_set(ctx, synth, 4096, 14336, 3, salt=200 + r) for r in range(n3)]
         d3 = [make_desc(capi, 3, 4096, 14336, 1, b) for b, _ in i3]
         verify(ctx, oracle, capi, d3[0], i3[0][1], 3, 4096, 14336, 1)
-        ms = timed_graph(ctx, [lambda d=d3[j % 8]: ctx.matmul(d) for j in range(160)]) / 160
-        wb = synth.weight_bytes(14336, 4096, bits=3)
+        ms = timed_graph(ctx, [lambda d=d3[j % n3]: ctx.matmul(d) for j in range(16 * n3)], reps=ROUNDS, rounds=True)[ROUNDS // 2] / (16 * n3)
         extra["gemv_int3_K4096_N14336"] = {"us": round(ms * 1e3, 3), "GB/s": round(wb / ms / 1e6, 1),
-                                           "hbm_frac": round(wb / ms / 1e6 / HBM_PEAK_GBS, 4)}
+                                           "hbm_frac": round(wb / ms / 1e6 / HBM_PEAK_GBS, 4), "rotation_MB": round(n3 * wb / 1e6, 1)}
         # 8-bit affine decode GEMV (int8_affine_matvec's shape family): twice the bytes per value, fewer vector
         # instructions per byte
         i8 = []
@@ -267,15 +367,16 @@ def main():
         ms = timed_graph(ctx, [lambda d=i8[j % 6]: ctx.matmul(d) for j in range(120)]) / 120
         wb = synth.weight_bytes(14336, 4096, bits=8)
         extra["gemv_int8_K4096_N14336"] = {"us": round(ms * 1e3, 3), "GB/s": round(wb / ms / 1e6, 1),
-                                           "hbm_frac": round(wb / ms / 1e6 / HBM_PEAK_GBS, 4)}
+                                           "hbm_frac": round(wb / ms / 1e6 / HBM_PEAK_GBS, 4), "rotation_MB": round(6 * wb / 1e6, 1)}
         # QKV matmul + RoPE + KV append in one dispatch at the configs[1] qkv shape (32 heads, 8 KV heads of 128 = 6144 rows)
         qs = []
         hps, vpo, kps = 16 * 128, 8 * 16 * 128, 2 * 8 * 16 * 128
         kvbuf, qout = ctx.alloc(64 * kps * 2), ctx.alloc(4096 * 2)
         ctx.fill(kvbuf, 0, 64 * kps * 2)
         pmap = _put(ctx, np.array([517], np.int32))
-        for r in range(8):
-            d0 = sets[r % args.sets][2]   # the (4096 -> 6144) weight set of the headline
+        nq = len(shape_sets[2])
+        for r in range(nq):
+            d0 = shape_sets[2][r]   # the (4096 -> 6144) weight sets of the headline
             qs.append(capi.QkvFusedDesc(bits=4, affine=1, k_packed=512, scales_per_row=64, heads=32, kv_heads=8, head_dim=128,
                                         page_size=16, kv_page_stride=kps, head_page_stride=hps, v_page_offset=vpo,
                                         rope_theta=500000.0, kv_capacity=64 * kps, q_out=qout, kv_pages=kvbuf, hidden=d0.in_,
@@ -283,10 +384,11 @@ def main():
         ctx.qkv_fused(qs[0])
         if not np.all(np.isfinite(ctx.download(qout, 4096 * 2, np.float16))):
             raise SystemExit("bench: fused QKV check failed")
-        ms = timed_graph(ctx, [lambda d=qs[j % 8]: ctx.qkv_fused(d) for j in range(160)]) / 160
+        ms = timed_graph(ctx, [lambda d=qs[j % nq]: ctx.qkv_fused(d) for j in range(8 * nq)]) / (8 * nq)
         wb = synth.weight_bytes(6144, 4096)
         extra["qkv_fused_rope_kvappend_K4096_N6144"] = {"us": round(ms * 1e3, 3), "GB/s": round(wb / ms / 1e6, 1),
-                                                        "hbm_frac": round(wb / ms / 1e6 / HBM_PEAK_GBS, 4)}
+                                                        "hbm_frac": round(wb / ms / 1e6 / HBM_PEAK_GBS, 4),
+                                                        "rotation_MB": round(nq * wb / 1e6, 1)}
         # the int8-KV pair at the same shape: QKV + RoPE to scratch rows, then the quantizer into the int8 pages
         kslot, vslot = ctx.alloc(1024 * 2), ctx.alloc(1024 * 2)
         i8pages, i8scales = ctx.alloc(64 * 8 * 16 * 2 * 32 * 4), ctx.alloc(64 * 8 * 16 * 2 * 2)
@@ -303,7 +405,7 @@ def main():
         krow = np.abs(ctx.download(kslot, 1024 * 2, np.float16).astype(np.float32)).reshape(8, 128).max(axis=1) / np.float32(127)
         if not np.array_equal(got_sc[:, 0], krow.astype(np.float16)):
             raise SystemExit("bench: int8 KV scale check failed")
-        ms2 = timed_graph(ctx, [lambda d=qs[j % 8]: int8_pair(d) for j in range(160)]) / 160
+        ms2 = timed_graph(ctx, [lambda d=qs[j % nq]: int8_pair(d) for j in range(8 * nq)]) / (8 * nq)
         ms1 = timed_graph(ctx, [lambda: ctx.kv_quantize_int8(kvq) for j in range(160)]) / 160
         extra["qkv_scratch_then_kv_quantize_int8_K4096_N6144"] = {"us": round(ms2 * 1e3, 3), "kv_quantize_us": round(ms1 * 1e3, 3)}
         # the four weight-streaming dispatches of one 8B decoder layer with the fused forms: QKV + RoPE + KV append,
@@ -313,12 +415,12 @@ def main():
             o_b, _ = upload_set(ctx, synth, 4096, 4096, 4, salt=500 + r)
             up_b, _ = upload_set(ctx, synth, 4096, 14336, 4, salt=520 + r)
             hbuf = ctx.alloc(14336 * 2)
-            g0, d0 = sets[r % args.sets][0], sets[r % args.sets][1]
+            g0, d0 = shape_sets[0][r % len(shape_sets[0])], shape_sets[1][r % len(shape_sets[1])]
             gated = capi.MatmulDesc(bits=4, affine=1, M=1, N=14336, k_packed=512, scales_per_row=64, out=hbuf, in_=g0.in_,
                                     scales=g0.scales, weights=g0.weights, biases=g0.biases)
             down = capi.MatmulDesc(bits=4, affine=1, M=1, N=4096, k_packed=1792, scales_per_row=224, out=d0.out, in_=hbuf,
                                    scales=d0.scales, weights=d0.weights, biases=d0.biases)
-            lsets.append((qs[r % 8], make_desc(capi, 4, 4096, 4096, 1, o_b), gated, (up_b["w"], up_b["s"], up_b["b"]), down))
+            lsets.append((qs[r % nq], make_desc(capi, 4, 4096, 4096, 1, o_b), gated, (up_b["w"], up_b["s"], up_b["b"]), down))
 
         def layer(L):
             q_, o_, g_, u_, d_ = L
@@ -332,7 +434,8 @@ def main():
         lbytes = (synth.weight_bytes(6144, 4096) + synth.weight_bytes(4096, 4096) + 2 * synth.weight_bytes(14336, 4096)
                   + synth.weight_bytes(4096, 14336))
         extra["decode_layer_8b_four_dispatches"] = {"us": round(ms * 1e3, 2), "GB/s": round(lbytes / ms / 1e6, 1),
-                                                    "hbm_frac": round(lbytes / ms / 1e6 / HBM_PEAK_GBS, 4), "weight_MB": round(lbytes / 1e6, 1)}
+                                                    "hbm_frac": round(lbytes / ms / 1e6 / HBM_PEAK_GBS, 4), "weight_MB": round(lbytes / 1e6, 1),
+                                                    "rotation_MB": round(6 * lbytes / 1e6, 1)}
         # gate + up + SiLU at the 8B layer shape, plain and with the add + RMSNorm prologue folded in
         dl, gm = _put(ctx, (synth.activations(1, 4096, salt=77).view(np.float16) * 0.3).astype(np.float16)), \
             _put(ctx, np.full(4096, 1.0, np.float16))
@@ -341,25 +444,31 @@ def main():
         gbytes = 2 * synth.weight_bytes(14336, 4096)
         extra["ffn_gated_K4096_N14336"] = {"us": round(ms_g * 1e3, 2), "GB/s": round(gbytes / ms_g / 1e6, 1),
                                            "hbm_frac": round(gbytes / ms_g / 1e6 / HBM_PEAK_GBS, 4),
-                                           "with_add_rmsnorm_prologue_us": round(ms_p * 1e3, 2)}
+                                           "with_add_rmsnorm_prologue_us": round(ms_p * 1e3, 2), "rotation_MB": round(6 * gbytes / 1e6, 1)}
         # small batches: the row-group GEMV (M <= 16) and the weight-streaming matrix-core kernel (M <= 128); int4,
         # configs[4]'s int3 M=8, and 8-bit rows (M=512: the 3-bit and 8-bit forms of the tile GEMM)
+        other_sets = {}
         for bits, M in ((4, 2), (4, 4), (4, 8), (4, 16), (4, 32), (4, 128), (3, 8), (3, 512), (8, 8), (8, 128), (8, 512)):
+            wb = synth.weight_bytes(14336, 4096, bits=bits)
             if bits == 4:
                 descs = [make_desc(capi, 4, 4096, 14336, M, b) for b, _ in gsets]
                 host0 = gsets[0][1]
             else:
-                other = [upload_set(ctx, synth, 4096, 14336, bits, salt=300 + 10 * bits + r, M=M) for r in range(3)]
+                if (bits, "sets") not in other_sets:   # one rotation per width, built for the largest M it is used at
+                    other_sets[(bits, "sets")] = [upload_set(ctx, synth, 4096, 14336, bits, salt=300 + 10 * bits + r, M=512)
+                                                  for r in range(n_sets(wb))]
+                other = other_sets[(bits, "sets")]
                 descs = [make_desc(capi, bits, 4096, 14336, M, b) for b, _ in other]
                 host0 = other[0][1]
+            nd = len(descs)
             verify(ctx, oracle, capi, descs[0], host0, bits, 4096, 14336, M)
             heavy = M >= 128  # matrix-core rows: sustained clock, as for the GEMM rows above
-            ms = timed_graph(ctx, [lambda d=descs[j % 3]: ctx.matmul(d) for j in range(36)], reps=6 if heavy else 1,
-                             warm=6 if heavy else 1) / 36
-            wb = synth.weight_bytes(14336, 4096, bits=bits)
+            ms = timed_graph(ctx, [lambda d=descs[j % nd]: ctx.matmul(d) for j in range(4 * nd)], reps=6 if heavy else 3,
+                             warm=6 if heavy else 1) / (4 * nd)
             extra["batch_int%d_M%d_K4096_N14336" % (bits, M)] = {
                 "us": round(ms * 1e3, 2), "TFLOP/s": round(2.0 * M * 4096 * 14336 / ms / 1e9, 1),
-                "weights_GB/s": round(wb / ms / 1e6, 1), "family": capi.KERNEL_NAMES[capi.resolve(descs[0])]}
+                "weights_GB/s": round(wb / ms / 1e6, 1), "family": capi.KERNEL_NAMES[capi.resolve(descs[0])],
+                "rotation_MB": round(nd * wb / 1e6, 1)}
         # MoE expert block (configs[3]): 256 experts, top-8, hidden 2048, intermediate 512; gate + up + down per token batch
         E, slots, d_model, ffn = 256, 8, 2048, 512
         moe_w = {}
@@ -368,26 +477,40 @@ def main():
             sc = synth.scales(N_, K_, experts=E, salt=len(name))
             bi = synth.biases(N_, K_, sc, experts=E, salt=len(name))
             moe_w[name] = tuple(_put(ctx, a) for a in (w, sc, bi))
+        per_expert = 2 * synth.weight_bytes(ffn, d_model) + synth.weight_bytes(d_model, ffn)
         for tokens in (1, 16):
-            ids = synth.topk_ids(tokens, slots, E, salt=tokens)
-            d_ids = _put(ctx, ids)
+            # every replay routes to other experts: one token walks a permutation of all 256 experts in 32 replays,
+            # sixteen tokens draw fresh ids per replay, so the experts touched across the rotation (the whole 453 MB
+            # stack) do not fit the last-level cache and expert_GB/s is an HBM figure
+            if tokens == 1:
+                perm = np.random.default_rng(23).permutation(E).astype(np.uint32)
+                id_sets = [perm[8 * r:8 * r + 8].reshape(1, slots) for r in range(E // slots)]
+            else:
+                id_sets = [synth.topk_ids(tokens, slots, E, salt=100 * tokens + r) for r in range(6)]
             x = _put(ctx, synth.activations(tokens, d_model, salt=5))
             gu = ctx.alloc(tokens * slots * 2 * ffn * 2)
             out = ctx.alloc(tokens * slots * d_model * 2)
-            gcommon = dict(bits=4, affine=1, M=1, N=ffn, k_packed=d_model // 8, scales_per_row=d_model // 64, slots=slots,
-                           tokens=tokens, in_slot_stride=0, out_slot_stride=2 * ffn, in_tok_stride=d_model,
-                           out_tok_stride=slots * 2 * ffn, ids_stride=slots, experts=E, in_=x, ids=d_ids)
-            dg = capi.MatmulDesc(out=gu, weights=moe_w["gate"][0], scales=moe_w["gate"][1], biases=moe_w["gate"][2], **gcommon)
-            du = capi.MatmulDesc(out=gu + ffn * 2, weights=moe_w["up"][0], scales=moe_w["up"][1], biases=moe_w["up"][2], **gcommon)
-            dd = capi.MatmulDesc(bits=4, affine=1, M=1, N=d_model, k_packed=ffn // 8, scales_per_row=ffn // 64, slots=slots,
-                                 tokens=tokens, in_slot_stride=2 * ffn, out_slot_stride=d_model, in_tok_stride=slots * 2 * ffn,
-                                 out_tok_stride=slots * d_model, ids_stride=slots, experts=E, out=out, in_=gu, ids=d_ids,
-                                 weights=moe_w["down"][0], scales=moe_w["down"][1], biases=moe_w["down"][2])
-            ms = timed_graph(ctx, [lambda d=d_: ctx.matmul(d) for _ in range(20) for d_ in (dg, du, dd)]) / 20
-            distinct = len(set(int(v) for v in ids.reshape(-1)))
-            per_expert = 2 * synth.weight_bytes(ffn, d_model) + synth.weight_bytes(d_model, ffn)
-            extra["moe_block_tokens%d" % tokens] = {"us": round(ms * 1e3, 2), "pairs": tokens * slots, "distinct_experts": distinct,
-                                                     "expert_GB/s": round(distinct * per_expert / ms / 1e6, 1)}
+            trios = []
+            for ids in id_sets:
+                d_ids = _put(ctx, ids)
+                gcommon = dict(bits=4, affine=1, M=1, N=ffn, k_packed=d_model // 8, scales_per_row=d_model // 64, slots=slots,
+                               tokens=tokens, in_slot_stride=0, out_slot_stride=2 * ffn, in_tok_stride=d_model,
+                               out_tok_stride=slots * 2 * ffn, ids_stride=slots, experts=E, in_=x, ids=d_ids)
+                dg = capi.MatmulDesc(out=gu, weights=moe_w["gate"][0], scales=moe_w["gate"][1], biases=moe_w["gate"][2], **gcommon)
+                du = capi.MatmulDesc(out=gu + ffn * 2, weights=moe_w["up"][0], scales=moe_w["up"][1], biases=moe_w["up"][2], **gcommon)
+                dd = capi.MatmulDesc(bits=4, affine=1, M=1, N=d_model, k_packed=ffn // 8, scales_per_row=ffn // 64, slots=slots,
+                                     tokens=tokens, in_slot_stride=2 * ffn, out_slot_stride=d_model, in_tok_stride=slots * 2 * ffn,
+                                     out_tok_stride=slots * d_model, ids_stride=slots, experts=E, out=out, in_=gu, ids=d_ids,
+                                     weights=moe_w["down"][0], scales=moe_w["down"][1], biases=moe_w["down"][2])
+                trios.append((dg, du, dd))
+            nrep = 2 * len(trios)
+            ms = timed_graph(ctx, [lambda d=d_: ctx.matmul(d) for r in range(nrep) for d_ in trios[r % len(trios)]], reps=3) / nrep
+            per_replay = [len(set(int(v) for v in ids.reshape(-1))) for ids in id_sets]
+            union = len(set(int(v) for ids in id_sets for v in ids.reshape(-1)))
+            distinct = float(np.mean(per_replay))
+            extra["moe_block_tokens%d" % tokens] = {"us": round(ms * 1e3, 2), "pairs": tokens * slots, "distinct_experts": round(distinct, 1),
+                                                     "expert_GB/s": round(distinct * per_expert / ms / 1e6, 1),
+                                                     "rotation_MB": round(union * per_expert / 1e6, 1)}
         # the whole routed FFN of configs[3] with a shared expert (257 stacked experts, 9 slots): router logits
         # (8-bit) -> softmax top-k -> gate, up -> silu_mul -> down -> combine, routed on the device
         E1, S = E + 1, slots + 1
@@ -405,77 +528,87 @@ def main():
         r_s = _put(ctx, r_sh)
         r_b = _put(ctx, (-127.5 * r_sh.astype(np.float32)).astype(np.float16))
         for tokens in (1, 16):
-            xh = synth.activations(tokens, d_model, salt=6)
-            x = _put(ctx, xh)
+            # other activations every replay, so the router sends every replay to other experts and the experts
+            # touched across the rotation outgrow the last-level cache
+            NX = 32 if tokens == 1 else 6
+            xbank = [_put(ctx, synth.activations(tokens, d_model, salt=600 + r)) for r in range(NX)]
             logits, ids, score = ctx.alloc(tokens * E1 * 4), ctx.alloc(tokens * S * 4), ctx.alloc(tokens * S * 4)
             gu, hbuf = ctx.alloc(tokens * S * 2 * ffn * 2), ctx.alloc(tokens * S * ffn * 2)
             dn, y = ctx.alloc(tokens * S * d_model * 2), ctx.alloc(tokens * d_model * 2)
+            h2buf, dn2, y2 = ctx.alloc(tokens * S * ffn * 2), ctx.alloc(tokens * S * d_model * 2), ctx.alloc(tokens * d_model * 2)
             common = dict(bits=4, affine=1, M=1, slots=S, tokens=tokens, ids_stride=S, experts=E1, ids=ids)
-            dg = capi.MatmulDesc(N=ffn, k_packed=d_model // 8, scales_per_row=d_model // 64, in_slot_stride=0,
-                                 out_slot_stride=2 * ffn, in_tok_stride=d_model, out_tok_stride=S * 2 * ffn, in_=x, out=gu,
-                                 weights=full_w["gate"][0], scales=full_w["gate"][1], biases=full_w["gate"][2], **common)
-            du = capi.MatmulDesc(N=ffn, k_packed=d_model // 8, scales_per_row=d_model // 64, in_slot_stride=0,
-                                 out_slot_stride=2 * ffn, in_tok_stride=d_model, out_tok_stride=S * 2 * ffn, in_=x,
-                                 out=gu + ffn * 2, weights=full_w["up"][0], scales=full_w["up"][1], biases=full_w["up"][2], **common)
             dd = capi.MatmulDesc(N=d_model, k_packed=ffn // 8, scales_per_row=ffn // 64, in_slot_stride=ffn,
                                  out_slot_stride=d_model, in_tok_stride=S * ffn, out_tok_stride=S * d_model, in_=hbuf, out=dn,
                                  weights=full_w["down"][0], scales=full_w["down"][1], biases=full_w["down"][2], **common)
-            ops = [("router_logits", lambda: ctx.moe_router_logits(logits, x, r_w, r_s, r_b, 8, d_model, E1, tokens)),
-                   ("router_topk", lambda: ctx.moe_router_topk(ids, score, logits, E, slots, True, True, tokens)),
-                   ("gate", lambda: ctx.matmul(dg)), ("up", lambda: ctx.matmul(du)),
-                   ("silu_mul", lambda: ctx.silu_mul(hbuf, gu, tokens * S, ffn)),
-                   ("down", lambda: ctx.matmul(dd)),
-                   ("combine", lambda: ctx.moe_combine(y, dn, score, tokens, d_model, S))]
-            for _, fn in ops:
-                fn()
-            # routing checked against the oracle before anything is timed
-            got_ids = ctx.download(ids, tokens * S * 4, np.uint32).reshape(tokens, S)
-            lg = ctx.download(logits, tokens * E1 * 4, np.float32).reshape(tokens, E1)
-            ref_ids, _ = oracle.router_topk(lg, tokens, E, slots, True, True)
-            yy = ctx.download(y, tokens * d_model * 2, np.float16)
-            if not np.array_equal(got_ids, ref_ids) or not np.all(np.isfinite(yy)):
-                raise SystemExit("bench: routed FFN check failed (tokens=%d)" % tokens)
-            ms = timed_graph(ctx, [fn for _ in range(20) for _, fn in ops]) / 20
-            row = {"us": round(ms * 1e3, 2), "dispatches": len(ops), "slots": S}
-            for name, fn in ops:
-                row[name + "_us"] = round(timed_graph(ctx, [fn] * 40) / 40 * 1e3, 2)
-            extra["moe_ffn_routed_tokens%d" % tokens] = row
-            # the same block in five launches: gate + up + SiLU in one pass over the activations
-            h2buf, dn2, y2 = ctx.alloc(tokens * S * ffn * 2), ctx.alloc(tokens * S * d_model * 2), ctx.alloc(tokens * d_model * 2)
-            dgated = capi.MatmulDesc(N=ffn, k_packed=d_model // 8, scales_per_row=d_model // 64, in_slot_stride=0,
-                                     out_slot_stride=ffn, in_tok_stride=d_model, out_tok_stride=S * ffn, in_=x, out=h2buf,
-                                     weights=full_w["gate"][0], scales=full_w["gate"][1], biases=full_w["gate"][2], **common)
             dd2 = capi.MatmulDesc(N=d_model, k_packed=ffn // 8, scales_per_row=ffn // 64, in_slot_stride=ffn,
                                   out_slot_stride=d_model, in_tok_stride=S * ffn, out_tok_stride=S * d_model, in_=h2buf, out=dn2,
                                   weights=full_w["down"][0], scales=full_w["down"][1], biases=full_w["down"][2], **common)
-            fused = [ops[0], ops[1],
-                     ("gate_up_silu", lambda: ctx.ffn_gated(dgated, full_w["up"][0], full_w["up"][1], full_w["up"][2])),
-                     ("down", lambda: ctx.matmul(dd2)),
-                     ("combine", lambda: ctx.moe_combine(y2, dn2, score, tokens, d_model, S))]
-            for _, fn in fused:
-                fn()
-            y_f = ctx.download(y2, tokens * d_model * 2, np.float16).astype(np.float64)
-            y_u = yy.astype(np.float64)
-            if (not np.array_equal(ctx.download(ids, tokens * S * 4, np.uint32).reshape(tokens, S), ref_ids)
-                    or float(np.max(np.abs(y_f - y_u)) / (np.max(np.abs(y_u)) + 1e-2)) > 1e-2):  # outputs cross zero: scale by the largest
-                raise SystemExit("bench: fused routed FFN disagrees with the seven-dispatch form (tokens=%d)" % tokens)
-            ms = timed_graph(ctx, [fn for _ in range(20) for _, fn in fused]) / 20
-            row = {"us": round(ms * 1e3, 2), "dispatches": len(fused), "slots": S}
-            for name, fn in fused:
-                row[name + "_us"] = round(timed_graph(ctx, [fn] * 40) / 40 * 1e3, 2)
-            extra["moe_ffn_routed_fused_tokens%d" % tokens] = row
+
+            def block(x):
+                gshape = dict(N=ffn, k_packed=d_model // 8, scales_per_row=d_model // 64, in_slot_stride=0, in_tok_stride=d_model, in_=x)
+                dg = capi.MatmulDesc(out_slot_stride=2 * ffn, out_tok_stride=S * 2 * ffn, out=gu, weights=full_w["gate"][0],
+                                     scales=full_w["gate"][1], biases=full_w["gate"][2], **gshape, **common)
+                du = capi.MatmulDesc(out_slot_stride=2 * ffn, out_tok_stride=S * 2 * ffn, out=gu + ffn * 2, weights=full_w["up"][0],
+                                     scales=full_w["up"][1], biases=full_w["up"][2], **gshape, **common)
+                dgated = capi.MatmulDesc(out_slot_stride=ffn, out_tok_stride=S * ffn, out=h2buf, weights=full_w["gate"][0],
+                                         scales=full_w["gate"][1], biases=full_w["gate"][2], **gshape, **common)
+                route = [("router_logits", lambda: ctx.moe_router_logits(logits, x, r_w, r_s, r_b, 8, d_model, E1, tokens)),
+                         ("router_topk", lambda: ctx.moe_router_topk(ids, score, logits, E, slots, True, True, tokens))]
+                seven = route + [("gate", lambda: ctx.matmul(dg)), ("up", lambda: ctx.matmul(du)),
+                                 ("silu_mul", lambda: ctx.silu_mul(hbuf, gu, tokens * S, ffn)),
+                                 ("down", lambda: ctx.matmul(dd)),
+                                 ("combine", lambda: ctx.moe_combine(y, dn, score, tokens, d_model, S))]
+                five = route + [("gate_up_silu", lambda: ctx.ffn_gated(dgated, full_w["up"][0], full_w["up"][1], full_w["up"][2])),
+                                ("down", lambda: ctx.matmul(dd2)),
+                                ("combine", lambda: ctx.moe_combine(y2, dn2, score, tokens, d_model, S))]
+                return seven, five
+
+            blocks = [block(x) for x in xbank]
+            touched = set()
+            for k, (seven, five) in enumerate(blocks):
+                for _, fn in seven:
+                    fn()
+                got_ids = ctx.download(ids, tokens * S * 4, np.uint32).reshape(tokens, S)
+                touched.update(int(v) for v in got_ids.reshape(-1))
+                if k == 0:
+                    # routing checked against the oracle before anything is timed, and the five-dispatch form against the seven
+                    lg = ctx.download(logits, tokens * E1 * 4, np.float32).reshape(tokens, E1)
+                    ref_ids, _ = oracle.router_topk(lg, tokens, E, slots, True, True)
+                    yy = ctx.download(y, tokens * d_model * 2, np.float16)
+                    if not np.array_equal(got_ids, ref_ids) or not np.all(np.isfinite(yy)):
+                        raise SystemExit("bench: routed FFN check failed (tokens=%d)" % tokens)
+                    for _, fn in five:
+                        fn()
+                    y_f = ctx.download(y2, tokens * d_model * 2, np.float16).astype(np.float64)
+                    y_u = yy.astype(np.float64)
+                    if (not np.array_equal(ctx.download(ids, tokens * S * 4, np.uint32).reshape(tokens, S), ref_ids)
+                            or float(np.max(np.abs(y_f - y_u)) / (np.max(np.abs(y_u)) + 1e-2)) > 1e-2):  # outputs cross zero: scale by the largest
+                        raise SystemExit("bench: fused routed FFN disagrees with the seven-dispatch form (tokens=%d)" % tokens)
+            rot_mb = round(len(touched) * per_expert / 1e6, 1)
+            for which, key in ((0, "moe_ffn_routed_tokens%d"), (1, "moe_ffn_routed_fused_tokens%d")):
+                lists = [b_[which] for b_ in blocks]
+                nrep = 2 * NX
+                ms = timed_graph(ctx, [fn for r in range(nrep) for _, fn in lists[r % NX]], reps=3) / nrep
+                row = {"us": round(ms * 1e3, 2), "dispatches": len(lists[0]), "slots": S, "rotation_MB": rot_mb}
+                for i_op, (name, _) in enumerate(lists[0]):
+                    # a dispatch alone, rotating over the same activations (the ids the router left last are the last set's:
+                    # the expert dispatches alone re-read one set of experts, so their solo times are lower bounds)
+                    row[name + "_us"] = round(timed_graph(ctx, [lists[r % NX][i_op][1] for r in range(2 * NX)]) / (2 * NX) * 1e3, 2)
+                extra[key % tokens] = row
         # elementwise / load-time kernels at their large shapes: HBM-bound, bytes moved per second
         rows_, f_ = 512, 14336
-        gu = ctx.alloc(rows_ * 2 * f_ * 2)
-        ho = ctx.alloc(rows_ * f_ * 2)
-        ctx.fill(gu, 0x3C, rows_ * 2 * f_ * 2)
-        ms = timed_graph(ctx, [lambda: ctx.silu_mul(ho, gu, rows_, f_)] * 20) / 20
-        extra["silu_mul_rows512_ffn14336"] = {"us": round(ms * 1e3, 2), "GB/s": round(rows_ * f_ * 6 / ms / 1e6, 1)}
+        nsl = n_sets(rows_ * f_ * 6)
+        gus, hos = [ctx.alloc(rows_ * 2 * f_ * 2) for _ in range(nsl)], [ctx.alloc(rows_ * f_ * 2) for _ in range(nsl)]
+        for g_ in gus:
+            ctx.fill(g_, 0x3C, rows_ * 2 * f_ * 2)
+        ms = timed_graph(ctx, [lambda j=j: ctx.silu_mul(hos[j % nsl], gus[j % nsl], rows_, f_) for j in range(3 * nsl)], reps=3) / (3 * nsl)
+        extra["silu_mul_rows512_ffn14336"] = {"us": round(ms * 1e3, 2), "GB/s": round(rows_ * f_ * 6 / ms / 1e6, 1),
+                                              "rotation_MB": round(nsl * rows_ * f_ * 6 / 1e6, 1)}
         nb = 256 << 20
         src_, dst_ = ctx.alloc(nb), ctx.alloc(nb)
         ctx.fill(src_, 0x3C, nb)
         ms = timed_graph(ctx, [lambda: ctx.repack_part(dst_, src_, nb, capi.CONVERT_BF16_F16, 0)] * 6) / 6
-        extra["repack_bf16_to_f16_256MiB"] = {"us": round(ms * 1e3, 1), "GB/s": round(2 * nb / ms / 1e6, 1)}
+        extra["repack_bf16_to_f16_256MiB"] = {"us": round(ms * 1e3, 1), "GB/s": round(2 * nb / ms / 1e6, 1), "rotation_MB": round(2 * nb / 1e6, 1)}
         result["extra"] = extra
 
     if not args.no_cpu:

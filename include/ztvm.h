@@ -147,6 +147,12 @@ ZTVM_API int ztvm_fill(ztvm_ctx* ctx, uint64_t dst, size_t dst_off, int byte, si
 /* copyBufferToBuffer (tests/kernels/gpu.mjs:107-110): device-to-device, ordered on the stream (a kernel,
  * so it may be recorded). Both addresses and the size must be multiples of 16 bytes. */
 ZTVM_API int ztvm_copy(ztvm_ctx* ctx, uint64_t dst, uint64_t src, size_t bytes);
+/* Measurement aid with no counterpart in the reference: a kernel that reads `bytes` bytes from src with 16-byte
+ * loads and does nothing else (sink: 4 bytes of device memory it practically never writes), ordered on the
+ * stream and recordable. Its time is the empirical ceiling a bandwidth-bound dispatch of that size is held
+ * against, measured in the same run and the same way as the dispatch (scripts/kernel-ab-ours.mjs:75-99 times
+ * its kernels against the device's streaming rate the same way). */
+ZTVM_API int ztvm_read_probe(ztvm_ctx* ctx, uint64_t src, size_t bytes, uint64_t sink);
 ZTVM_API int ztvm_sync(ztvm_ctx* ctx);
 
 /* ---- dispatch ----------------------------------------------------------- */

@@ -68,6 +68,7 @@ hipError_t launch_gemm(const MatmulArgs& a, const Tune& t, void* scratch, hipStr
 size_t gemm_scratch_bytes(const MatmulArgs& a);
 hipError_t launch_dequant(const MatmulArgs& a, hipStream_t s);
 hipError_t launch_copy(void* dst, const void* src, size_t bytes, hipStream_t s);
+hipError_t launch_read_probe(const void* src, size_t bytes, void* sink, hipStream_t s);
 hipError_t launch_fill(void* dst, int byte, size_t bytes, hipStream_t s);
 
 // the dispatches around the matmuls of an FFN / MoE block (block_ops.hip)

@@ -368,6 +368,14 @@ int ztvm_copy(ztvm_ctx* ctx, uint64_t dst, uint64_t src, size_t bytes) {
   return ZTVM_OK;
 }
 
+int ztvm_read_probe(ztvm_ctx* ctx, uint64_t src, size_t bytes, uint64_t sink) {
+  if (!ctx || !src || !sink) return fail(ctx, ZTVM_E_INVALID, "ztvm_read_probe: null argument");
+  if ((src & 15u) || (bytes & 15u) || (sink & 3u)) return fail(ctx, ZTVM_E_INVALID, "ztvm_read_probe: src and size must be multiples of 16 bytes, sink of 4");
+  if (!bytes) return ZTVM_OK;
+  HIP_TRY(ctx, launch_read_probe(reinterpret_cast<const void*>(src), bytes, reinterpret_cast<void*>(sink), ctx->stream));
+  return ZTVM_OK;
+}
+
 int ztvm_sync(ztvm_ctx* ctx) {
   if (!ctx) return fail(nullptr, ZTVM_E_INVALID, "null context");
   if (ctx->recording) return fail(ctx, ZTVM_E_INVALID, "ztvm_sync while recording a command buffer");

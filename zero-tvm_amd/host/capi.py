@@ -15,7 +15,7 @@ E_INVALID, E_HIP, E_UNSUPPORTED, E_NODEVICE = -1, -2, -3, -4
 
 EXPORTS = [
     "ztvm_abi_version", "ztvm_last_error", "ztvm_create", "ztvm_destroy", "ztvm_device_info",
-    "ztvm_alloc", "ztvm_free", "ztvm_upload", "ztvm_download", "ztvm_fill", "ztvm_copy", "ztvm_sync",
+    "ztvm_alloc", "ztvm_free", "ztvm_upload", "ztvm_download", "ztvm_fill", "ztvm_copy", "ztvm_read_probe", "ztvm_sync",
     "ztvm_matmul_validate", "ztvm_matmul_resolve", "ztvm_matmul", "ztvm_matmul_static", "ztvm_ffn_gated", "ztvm_ffn_gated_prologue", "ztvm_qkv_fused", "ztvm_qkv_fused_scratch",
     "ztvm_kv_quantize_int8", "ztvm_dequant",
     "ztvm_record_begin", "ztvm_record_end", "ztvm_submit", "ztvm_cmdbuf_destroy",
@@ -83,6 +83,7 @@ def load():
     L.ztvm_download.argtypes = [vp, vp, C.c_uint64, C.c_size_t, C.c_size_t]
     L.ztvm_fill.argtypes = [vp, C.c_uint64, C.c_size_t, C.c_int, C.c_size_t]
     L.ztvm_copy.argtypes = [vp, C.c_uint64, C.c_uint64, C.c_size_t]
+    L.ztvm_read_probe.argtypes = [vp, C.c_uint64, C.c_size_t, C.c_uint64]
     L.ztvm_sync.argtypes = [vp]
     L.ztvm_matmul_validate.argtypes = [C.POINTER(MatmulDesc), C.c_char_p, C.c_size_t]
     L.ztvm_matmul_resolve.argtypes = [C.POINTER(MatmulDesc)]
@@ -189,6 +190,10 @@ class Context:
 
     def copy(self, dst, src, nbytes):
         self._chk(self._L.ztvm_copy(self._h, dst, src, nbytes))
+
+    def read_probe(self, src, nbytes, sink):
+        """A kernel that only reads nbytes from src: the streaming rate of the memory system, timed like a dispatch."""
+        self._chk(self._L.ztvm_read_probe(self._h, src, nbytes, sink))
 
     def sync(self):
         self._chk(self._L.ztvm_sync(self._h))
