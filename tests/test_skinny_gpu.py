@@ -46,17 +46,25 @@ CASES = [(2, 8, 64, 2560), (6, 8, 64, 2560), (31, 64, 256, 2560), (33, 64, 256, 
 @pytest.mark.parametrize("bits,affine", FORMATS)
 def test_ragged_skinny(ctx, capi, synth, oracle, M, CAP, N, K, bits, affine):
     A, w, s, b = make(synth, bits, affine, CAP, N, K)
-    ctx.set_option("skinny.ksplit", 1)  # one summation order whatever M is
+    ref = oracle.gemm(oracle.MODE_FORMULA_F64, bits, affine, M, N, K, A, w, s, b, threads=8)
+
+    def check(got):
+        y = got[:M].view(np.float16).astype(np.float64)
+        assert rel_err(y, ref, 1e-2) < 1e-2
+        assert rel_err(y, ref, 1e-3) < 2e-2
+        assert not got[M:].any(), "rows past M were written"
+
+    check(run(ctx, capi, bits, affine, M, CAP, N, K, A, w, s, b, capi.KERNEL_SKINNY))  # the tile shape and k split chosen for M
+    # one tile shape and one k split whatever M is: a row's bits must not depend on the rows that travel with it
+    ctx.set_option("skinny.ksplit", 1)
+    ctx.set_option("skinny.shape", 2)
     try:
         got = run(ctx, capi, bits, affine, M, CAP, N, K, A, w, s, b, capi.KERNEL_SKINNY)
         gotcap = run(ctx, capi, bits, affine, CAP, CAP, N, K, A, w, s, b, capi.KERNEL_SKINNY)
     finally:
         ctx.set_option("skinny.ksplit", 0)
-    y = got[:M].view(np.float16).astype(np.float64)
-    ref = oracle.gemm(oracle.MODE_FORMULA_F64, bits, affine, M, N, K, A, w, s, b, threads=8)
-    assert rel_err(y, ref, 1e-2) < 1e-2
-    assert rel_err(y, ref, 1e-3) < 2e-2
-    assert not got[M:].any(), "rows past M were written"
+        ctx.set_option("skinny.shape", 0)
+    check(got)
     assert np.array_equal(got[:M], gotcap[:M]), "M-variance"
 
 

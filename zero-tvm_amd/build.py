@@ -12,7 +12,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libztvm_hip.so")
-SOURCES = ["ztvm_api.hip", "gemv.hip", "gemv_stream.hip", "gemv_rows.hip", "skinny.hip", "gemm.hip", "dequant.hip", "block_ops.hip", "repack.hip"]
+SOURCES = ["ztvm_api.hip", "gemv.hip", "gemv_stream.hip", "gemv_rows.hip", "skinny.hip", "skinny_dma.hip", "gemm.hip", "dequant.hip", "block_ops.hip", "repack.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC", "-fvisibility=hidden",

@@ -28,25 +28,10 @@
 // reference's kernel for it: K_PACKED = K/4, four values per word).
 #include "internal.h"
 #include "mma.h"
+#include "skinny.h"
 
 namespace ztvm {
 namespace {
-
-constexpr int KS = 64;             // k per step
-constexpr int WAVES = 4;           // waves per workgroup = 128 output columns
-
-struct StreamParams {
-  void* out;
-  const _Float16* inp;   // activations, chunks of 8 in slot order
-  const _Float16* scales;
-  const uint32_t* weights;
-  const _Float16* biases;
-  const _Float16* xs16;  // [M][xs_stride]: hi halves, lo halves of the group sums, zero padding
-  uint32_t M, N, K, row_words, spr;
-  uint32_t nsteps, bias_steps, xs_stride, mtiles, ngroups, out_f32, xcd_swizzle;
-  uint32_t ksplit, steps_per_split;  // k steps are dealt to ksplit workgroups, steps_per_split each
-  float* partial;                    // [ksplit][M][N] when ksplit > 1
-};
 
 // Pre-pass: slot-ordered copy of the activations and, for affine weights, the group sums
 // xs16[m][g] = f16(xs), xs16[m][G+g] = f16(xs - hi), zero from 2G up to the stride.
@@ -94,6 +79,17 @@ struct WRegs {
   uint32_t s;  // one f16 scale (affine) or two (symmetric)
 };
 
+// step(0); if more(1) { step(1); if more(2) { ... } }, entered only if more(0)
+template <int J, int N, class More, class Step>
+__device__ __forceinline__ void nested_for(More&& more, Step&& step) {
+  if constexpr (J < N) {
+    if (more(J)) {
+      step(std::integral_constant<int, J>{});
+      nested_for<J + 1, N>(more, step);
+    }
+  }
+}
+
 // MB: 32-row blocks of the activation tile. CLAMP: the tile is taller than M, rows past M repeat
 // row M-1; otherwise a partial last tile is moved up to end at row M.
 //
@@ -101,8 +97,12 @@ struct WRegs {
 // waits carry exact counts: the packed weights, scales and the activation tile of step s+DEPTH
 // are fetched into registers while step s computes (DEPTH steps of latency hidden per wave),
 // the activation registers of step s are written to one of two LDS buffers, one barrier per step.
+//
+// The weight loads are ordinary cached loads: a lane's 16 bytes of step s and the 16 of its lane half partner are
+// 32 consecutive bytes of a weight row, so a 128-byte line serves four steps and must stay in the vector cache for
+// them (with the streaming hint every step asked the second-level cache again: 2.6 M requests a launch at 32 rows
+// against 1.5 M without, 31 us against 27).
 constexpr int DEPTH = 4;
-
 template <int MB, int BITS, bool AFFINE, bool CLAMP>
 __global__ __launch_bounds__(64 * WAVES) void stream_kernel(const StreamParams p) {
   static_assert(BITS == 4 || ((BITS == 3 || BITS == 8) && AFFINE), "formats");
@@ -157,11 +157,12 @@ __global__ __launch_bounds__(64 * WAVES) void stream_kernel(const StreamParams p
   struct ARegs {
     u32x4 v[MB];
   };
-  auto fetch_a = [&](ARegs& a, const _Float16** src) __attribute__((always_inline)) {
+  // adv: elements to advance by afterwards (0 once the last step of the range has been fetched)
+  auto fetch_a = [&](ARegs& a, const _Float16** src, uint32_t adv) __attribute__((always_inline)) {
 #pragma unroll
     for (int r = 0; r < MB; r++) {
       a.v[r] = *reinterpret_cast<const u32x4*>(src[r]);
-      src[r] += KS;
+      src[r] += adv;
     }
   };
   auto store_a = [&](const ARegs& a, uint32_t buf) __attribute__((always_inline)) {
@@ -172,18 +173,20 @@ __global__ __launch_bounds__(64 * WAVES) void stream_kernel(const StreamParams p
   // ---- weights and scales of this lane's column
   const uint32_t* w_src = p.weights + (size_t)n * p.row_words + (size_t)s_begin * W_STEP_WORDS + (BITS == 3 ? h * 3 : (BITS == 8 ? h * 8 : (AFFINE ? h * 4 : 0)));
   const _Float16* sc_src = p.scales + (size_t)n * p.spr + (size_t)s_begin * RPB;
-  auto fetch_w = [&](WRegs& r) __attribute__((always_inline)) {
+  uint32_t sc_tie = 0;  // always 0, but the compiler must not know
+  asm volatile("" : "+v"(sc_tie));
+  auto fetch_w = [&](WRegs& r, bool adv) __attribute__((always_inline)) {
     if constexpr (BITS == 3) {
-      const u32x3_a4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x3_a4*>(w_src));
+      const u32x3_a4 v = *reinterpret_cast<const u32x3_a4*>(w_src);
       r.c = (u32x3){v.x, v.y, v.z};
     } else {
-      r.a = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(w_src));
-      if constexpr (!AFFINE || BITS == 8) r.b = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(w_src + 4));
+      r.a = *reinterpret_cast<const u32x4*>(w_src);
+      if constexpr (!AFFINE || BITS == 8) r.b = *reinterpret_cast<const u32x4*>(w_src + 4);
     }
-    if constexpr (AFFINE) r.s = *reinterpret_cast<const uint16_t*>(sc_src);
-    else r.s = *reinterpret_cast<const uint32_t*>(sc_src);
-    w_src += W_STEP_WORDS;
-    sc_src += RPB;
+    if constexpr (AFFINE) r.s = *reinterpret_cast<const uint16_t*>(sc_src + sc_tie);
+    else r.s = *reinterpret_cast<const uint32_t*>(sc_src + sc_tie);
+    w_src += adv ? W_STEP_WORDS : 0;
+    sc_src += adv ? RPB : 0;
   };
   // MFMA t of a step multiplies k chunk chunk_of(t) of the step: both 8-k halves of an MFMA
   // (lane halves h) must lie in one group
@@ -245,7 +248,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_kernel(const StreamParams p
     const _Float16* brow = p.biases + (size_t)n * G;
     for (uint32_t bs = 0; bs < p.bias_steps; bs++) {
       ARegs xa;
-      fetch_a(xa, xs_src);
+      fetch_a(xa, xs_src, KS);
       h8 bf[4];
 #pragma unroll
       for (int t = 0; t < 4; t++) {
@@ -282,10 +285,18 @@ __global__ __launch_bounds__(64 * WAVES) void stream_kernel(const StreamParams p
   part[1] = zero;
 
 
-  // one step: position j in the ring; REFILL: the ring slot is refilled for step s+DEPTH
-  auto step = [&](auto jc, auto refill_c) __attribute__((always_inline)) {
+  // Steps fetched so far. Every step refills its ring slot with step s+DEPTH: past the end of the range the
+  // fetch repeats the last step (the pointers stop advancing) and nobody reads the result, so the loop has one
+  // shape for every range length and no wait of it ever has to allow for a path with fewer loads in flight.
+  uint32_t fetched = 0;
+  auto fetch = [&](int j) __attribute__((always_inline)) {
+    const bool adv = ++fetched < nsteps;
+    fetch_w(wq[j], adv);
+    fetch_a(aq[j], a_src, adv ? KS : 0);
+  };
+  // one step: position j in the ring
+  auto step = [&](auto jc) __attribute__((always_inline)) {
     constexpr int j = decltype(jc)::value;
-    constexpr bool REFILL = decltype(refill_c)::value;
     constexpr uint32_t buf = j & 1;
     // this step's activations into LDS, its weights into the B operands
     store_a(aq[j], buf);
@@ -293,10 +304,14 @@ __global__ __launch_bounds__(64 * WAVES) void stream_kernel(const StreamParams p
     for (int t = 0; t < 4; t++) Bf[t] = unpack_t(wq[j], t);
 #pragma unroll
     for (int g = 0; g < RPB; g++) sc_cur[g] = scale_of(wq[j], g);
-    if (REFILL) {
-      fetch_w(wq[j]);
-      fetch_a(aq[j], a_src);
-    }
+    // The scale must be a float before its ring slot is refilled. Left alone the compiler folds the
+    // conversion into the FMAs of the NEXT step, keeps the raw halfword alive past the refill, and pays for
+    // that with register copies of values still in flight at the top of the loop, where waiting for them
+    // drains the ring. The empty statement makes the refill's address (sc_src + sc_tie, sc_tie always 0)
+    // depend on the converted value.
+#pragma unroll
+    for (int g = 0; g < RPB; g++) asm volatile("" : "+v"(sc_cur[g]), "+v"(sc_tie));
+    fetch(j);
     __syncthreads();
 #pragma unroll
     for (int t = 0; t < 4; t++) Af[0][t] = read_a(buf, 0, t);
@@ -324,38 +339,13 @@ __global__ __launch_bounds__(64 * WAVES) void stream_kernel(const StreamParams p
     sc_prev = sc_cur[RPB - 1];
     if (NRUN % 2) part[1] = part[0];  // the next step folds part[1] first
   };
-  using yes = std::integral_constant<bool, true>;
-  using no = std::integral_constant<bool, false>;
-  // groups of DEPTH steps whose refills are all in range: no branches, exact wait counts. The ring is
-  // primed on a path of its own: a wait count is fixed per instruction, so the loop's waits can only be
-  // as loose as the tightest path that reaches the loop, and a priming sequence with a branch per slot
-  // (short k ranges) would have every wait in the loop drain all loads in flight.
-  uint32_t s = 0;
-  if (nsteps >= 2 * DEPTH) {
-    static_for<DEPTH>([&](auto jc) {
-      constexpr int j = decltype(jc)::value;
-      fetch_w(wq[j]);
-      fetch_a(aq[j], a_src);
-    });
-    for (; s + 2 * DEPTH <= nsteps; s += DEPTH) static_for<DEPTH>([&](auto jc) { step(jc, yes{}); });
-  } else {
-    static_for<DEPTH>([&](auto jc) {
-      constexpr int j = decltype(jc)::value;
-      if (j < nsteps) {
-        fetch_w(wq[j]);
-        fetch_a(aq[j], a_src);
-      }
-    });
-  }
-  // up to 2*DEPTH - 1 remaining steps
-  for (; s < nsteps; s += DEPTH) {
-    static_for<DEPTH>([&](auto jc) {
-      constexpr int j = decltype(jc)::value;
-      if (s + j < nsteps) {
-        if (s + j + DEPTH < nsteps) step(jc, yes{});
-        else step(jc, no{});
-      }
-    });
+  if (nsteps > 0) {
+    static_for<DEPTH>([&](auto jc) { fetch(decltype(jc)::value); });
+    // whole turns of the ring, then the rest as nested conditions: a step that is not reached leaves for the
+    // end of the kernel, so no step is ever entered from a path that skipped the one before it
+    uint32_t s = 0;
+    for (; s + DEPTH <= nsteps; s += DEPTH) static_for<DEPTH>(step);
+    nested_for<0, DEPTH - 1>([&](int j) { return s + j < nsteps; }, step);
   }
   // the last run is still unfolded
   if (nsteps > 0) {
@@ -411,9 +401,9 @@ hipError_t launch_fmt(const StreamParams& p, int mb, hipStream_t s) {
   return launch_mb<4, BITS, AFFINE>(p, s);
 }
 
-uint32_t xs_stride_of(const MatmulArgs& a) { return a.affine ? (2 * a.spr + KS - 1) / KS * KS : 0; }
-
 int blocks_of(uint32_t M) { return M <= 32 ? 1 : (M <= 64 ? 2 : 4); }
+
+uint32_t xs_stride_of(const MatmulArgs& a) { return a.affine ? (2 * a.spr + KS - 1) / KS * KS : 0; }
 
 // k splits: one round of workgroups over the CUs for a single row tile (measured: 2 beats 3 at 112
 // column groups on 256 CUs, 8 wins at 32 groups). A function of N and K only, so that a row's
@@ -449,7 +439,7 @@ bool skinny_supports(const MatmulArgs& a) {
 }
 
 size_t skinny_scratch_bytes(const MatmulArgs& a, const Tune& t) {
-  const uint32_t ks = ksplit_of(a, t);
+  const uint32_t ks = skinny_dma_supports(a, t) ? skinny_dma_ksplit(a, t) : ksplit_of(a, t);
   return align256((size_t)a.M * a.K * sizeof(_Float16)) + align256((size_t)a.M * xs_stride_of(a) * sizeof(_Float16)) +
          (ks > 1 ? align256((size_t)ks * a.M * a.N * sizeof(float)) : 0) + 256;
 }
@@ -471,11 +461,14 @@ hipError_t launch_skinny(const MatmulArgs& a, const Tune& t, void* scratch, hipS
   p.xs_stride = xs_stride_of(a);
   p.bias_steps = a.affine ? p.xs_stride / KS : 0;
   p.xcd_swizzle = t.gemm_xcd_swizzle;
+  const bool dma = skinny_dma_supports(a, t);
   const int mb = blocks_of(a.M);
-  p.mtiles = (a.M + 32 * mb - 1) / (32 * mb);
-  p.ngroups = (a.N + 32 * WAVES - 1) / (32 * WAVES);
-  p.ksplit = ksplit_of(a, t);
-  p.steps_per_split = (p.nsteps + p.ksplit - 1) / p.ksplit;
+  if (!dma) {
+    p.mtiles = (a.M + 32 * mb - 1) / (32 * mb);
+    p.ngroups = (a.N + 32 * WAVES - 1) / (32 * WAVES);
+    p.ksplit = ksplit_of(a, t);
+    p.steps_per_split = (p.nsteps + p.ksplit - 1) / p.ksplit;
+  }
   {
     const uint32_t pad = a.affine ? p.xs_stride - 2 * (a.K / 64) : 0, cpr = a.K / 8;
     const uint32_t nthr = a.M * (cpr > pad ? cpr : pad);  // one thread per chunk, and enough for the padding columns
@@ -483,7 +476,8 @@ hipError_t launch_skinny(const MatmulArgs& a, const Tune& t, void* scratch, hipS
                        (uint32_t)(a.bits == 8));
   }
   hipError_t e;
-  if (a.bits == 3) e = launch_fmt<3, true>(p, mb, s);
+  if (dma) e = launch_skinny_dma(p, a, t, s);
+  else if (a.bits == 3) e = launch_fmt<3, true>(p, mb, s);
   else if (a.bits == 8) e = launch_fmt<8, true>(p, mb, s);
   else if (a.affine) e = launch_fmt<4, true>(p, mb, s);
   else e = launch_fmt<4, false>(p, mb, s);

@@ -248,6 +248,8 @@ const Option kOptions[] = {
     {"gemv.stream", &Tune::gemv_stream},
     {"gemv.ring", &Tune::gemv_ring},
     {"skinny.ksplit", &Tune::skinny_ksplit},
+    {"skinny.dma", &Tune::skinny_dma},
+    {"skinny.shape", &Tune::skinny_shape},
     {"rows.wg_per_cu", &Tune::rows_wg_per_cu},
     {"rows.waves", &Tune::rows_waves},
     {"gemm.tile", &Tune::gemm_tile},
