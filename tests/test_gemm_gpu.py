@@ -57,11 +57,13 @@ def test_ragged_gemm(ctx, capi, synth, oracle, M, CAP, N, K, affine, family):
         return capi.resolve(capi.MatmulDesc(bits=4, affine=int(affine), kernel=kernel, M=m, N=N, k_packed=K // 8,
                                             scales_per_row=K // (64 if affine else 32), out=4096, in_=4096, scales=4096,
                                             weights=4096, biases=4096 if affine else 0))
-    if family_of(M) == family_of(CAP):
+    # the skinny family has two tile shapes (up to 32 rows, above) that deal K to their waves differently
+    same_order = family_of(M) == family_of(CAP) and not (family_of(M) == capi.KERNEL_SKINNY and (M <= 32) != (CAP <= 32))
+    if same_order:
         assert np.array_equal(got[:M], gotcap[:M]), "M-variance"
     else:
-        # AUTO changes family with M (2, 17 and 129 rows): a row's result is bit-stable inside a family; across
-        # families it agrees to the last f16 bit or two (different f32 summation order)
+        # AUTO changes family with M (2, 17 and 129 rows): a row's result is bit-stable inside a family and tile shape;
+        # across them it agrees to the last f16 bit or two (different f32 summation order)
         assert rel_err(y, gotcap[:M].view(np.float16).astype(np.float64), 1e-2) < 2e-3
 
 

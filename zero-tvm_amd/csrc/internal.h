@@ -51,7 +51,7 @@ struct Tune {
   int gemv_ring = 0;        // passes in flight per wave of the streaming kernel (0: two; 1, 3)
   int gemv_stream = 0;      // 0: dense single rows go to the register-resident streaming kernel where it applies; 1: never
   int skinny_dma = 0;        // 1: the transfer-engine form of the skinny kernel is switched off
-  int skinny_shape = 0;      // transfer-engine form: 0 = by M; 1 = 32 rows x 128 columns x 4 k parts; 2 = 64 x 128 x 2; 3 = 32 x 64 x 4
+  int skinny_shape = 0;      // transfer-engine form: 0 = by M; 2 = 64 rows x 128 columns x 2 k parts; 3 = 32 x 64 x 4
   int skinny_ksplit = 0;     // workgroups sharing the k range of one skinny tile (0: chosen from M, N, K)
   int rows_wg_per_cu = 0;    // the row-group GEMV: workgroups per CU and waves per workgroup (0: chosen from the LDS it stages)
   int rows_waves = 0;

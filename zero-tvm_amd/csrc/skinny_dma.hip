@@ -10,8 +10,13 @@
 //     and asked for twice; the scales were asked for once per step, 2 bytes out of 64;
 //   * the workgroup is NW column waves (32 output columns each) times KH k parts. Each k part runs its own pipeline
 //     over its own share of K; the parts meet at one barrier per unit and add their totals through LDS at the end, in
-//     part order. Two or more waves per SIMD: while one waits at the barrier or for its fragments another multiplies.
+//     part order. Two waves per SIMD: while one waits at the barrier or for its fragments the other multiplies.
 //     (One wave per SIMD, as in stream_kernel, spends its time waiting: 40% of the issue slots at 128 rows.)
+//
+// Measured at K=4096, N=14336 with per-turn time stamps: the waits for the transfers are empty (76 ticks of a 2400-tick
+// turn), so neither a deeper pipeline nor a wave that touches the weights ahead of time into the second-level cache
+// changes anything (both tried). A turn is the matrix and vector instructions of its two steps: 16 matrix and about
+// 150 vector instructions per wave at 64 rows, two waves per SIMD.
 //
 // Unit = two k steps = 128 k. LDS of k part p, stage t (D stages):
 //     activations  2 x ROWS x 128 B   step j at j*ROWS*128; row r = 8 chunks of 16 B, chunk c at (c ^ swz(r))
@@ -71,11 +76,12 @@ __global__ __launch_bounds__(64 * NW * KH) void dma_kernel(const StreamParams p)
   // ---- units of this workgroup, of this k part. steps_per_split is even; a part may come out empty.
   const uint32_t nunits = p.nsteps / 2, ups = p.steps_per_split / 2;
   const uint32_t u_begin = split * ups, u_stop = u_begin + ups < nunits ? u_begin + ups : nunits;  // u_begin < u_stop
-  const uint32_t upp = (u_stop - u_begin + KH - 1) / KH;  // turns of the loop, the same for every part
-  const uint32_t pu0 = u_begin + part * upp < u_stop ? u_begin + part * upp : u_stop;
-  const uint32_t pu1 = pu0 + upp < u_stop ? pu0 + upp : u_stop;
-  const uint32_t my_units = pu1 - pu0;
-  const uint32_t u_last = my_units ? pu1 - 1 : u_begin;  // fetches past the part's share repeat this unit; nobody reads them
+  const uint32_t nsplit = u_stop - u_begin;
+  const uint32_t upp = (nsplit + KH - 1) / KH;  // turns of the loop, the same for every part
+  // Part p multiplies units u_begin + p, u_begin + p + KH, ...: in one turn the KH parts fetch KH consecutive units,
+  // 64*KH consecutive bytes of every weight row.
+  const uint32_t my_units = part < nsplit ? (nsplit - part + KH - 1) / KH : 0;
+  const uint32_t u_last = u_stop - 1;  // fetches past the part's share repeat the split's last unit; nobody reads them
 
   // ---- transfers. Piece q = r*T + tp of a step's activation tile is LDS bytes [16q, 16q+16): row q/8, chunk slot q%8.
   uint32_t a_off[AP];
@@ -101,21 +107,35 @@ __global__ __launch_bounds__(64 * NW * KH) void dma_kernel(const StreamParams p)
   ncol = ncol < p.N ? ncol : p.N - 1;
   const uint32_t s_off = (ncol * p.spr + (AFFINE ? 0u : 2u * h)) * 2u;
   const uint32_t lds_part = lds0 + part * PART;
-  // unit u of this part's sequence (pu0 + i) into stage t
-  auto issue = [&](uint32_t i, uint32_t t) __attribute__((always_inline)) {
-    uint32_t u = pu0 + i;
+  // Transfer k (0 .. L-1) of unit i of this part's sequence, into stage t: the activations of step 0, of step 1, the
+  // weights, the scales.
+  auto issue_one = [&](auto kc, uint32_t i, uint32_t t) __attribute__((always_inline)) {
+    constexpr int k = decltype(kc)::value;
+    uint32_t u = u_begin + i * KH + part;
     u = u < u_last ? u : u_last;
-    const char* ab = reinterpret_cast<const char*>(p.inp) + (size_t)u * 256;
-    const char* wb = reinterpret_cast<const char*>(p.weights) + (size_t)u * 64;
-    const char* sb = reinterpret_cast<const char*>(p.scales) + (size_t)u * (AFFINE ? 4 : 8);
     const uint32_t st = lds_part + t * STAGE;
-#pragma unroll
-    for (int j = 0; j < 2; j++)
-#pragma unroll
-      for (int r = 0; r < AP; r++) dma16<0>(ab + j * 128, a_off[r], st + j * A_STEP + (r * NW + wc) * 1024u);
-#pragma unroll
-    for (int r = 0; r < 2; r++) dma16<0>(wb, w_off[r], st + A_BYTES + (r * NW + wc) * 1024u);
-    dma4(sb, s_off, st + A_BYTES + W_BYTES + wc * 256u);
+    if constexpr (k < 2 * AP) {
+      constexpr int j = k / AP, r = k % AP;
+      dma16<0>(reinterpret_cast<const char*>(p.inp) + (size_t)u * 256 + j * 128, a_off[r], st + j * A_STEP + (r * NW + wc) * 1024u);
+    } else if constexpr (k < 2 * AP + 2) {
+      constexpr int r = k - 2 * AP;
+      dma16<0>(reinterpret_cast<const char*>(p.weights) + (size_t)u * 64, w_off[r], st + A_BYTES + (r * NW + wc) * 1024u);
+    } else {
+      dma4(reinterpret_cast<const char*>(p.scales) + (size_t)u * (AFFINE ? 4 : 8), s_off, st + A_BYTES + W_BYTES + wc * 256u);
+    }
+  };
+  // transfers [L*slot/NSLOT, L*(slot+1)/NSLOT): a turn sends its L transfers in NSLOT helpings, between its runs of
+  // matrix instructions. Sent all at once after the barrier, every wave of the workgroup stood in the same queue
+  // (48 KB go through the vector cache at 64 bytes a clock) and none of them multiplied meanwhile: 0.3 to 0.7 us of a
+  // 2.1 us turn at 128 rows.
+  constexpr int NSLOT = 2 * NRUN;
+  auto issue_slot = [&](auto sc_, uint32_t i, uint32_t t) __attribute__((always_inline)) {
+    constexpr int slot = decltype(sc_)::value;
+    constexpr int k0 = L * slot / NSLOT, k1 = L * (slot + 1) / NSLOT;
+    static_for<k1 - k0>([&](auto kc) { issue_one(ic<k0 + decltype(kc)::value>{}, i, t); });
+  };
+  auto issue = [&](uint32_t i, uint32_t t) __attribute__((always_inline)) {
+    static_for<L>([&](auto kc) { issue_one(kc, i, t); });
   };
 
   UnpackConsts uc;
@@ -200,7 +220,9 @@ __global__ __launch_bounds__(64 * NW * KH) void dma_kernel(const StreamParams p)
   acc[0] = zero;
   acc[1] = zero;
   // one k step out of stage t of this part: j = 0, 1
-  auto step = [&](uint32_t st, int j) __attribute__((always_inline)) {
+  // (jc: step 0 or 1 of the unit; the turn's transfers for unit i_next go out between the runs)
+  auto step = [&](uint32_t st, auto jc, uint32_t i_next, uint32_t t_next) __attribute__((always_inline)) {
+    constexpr int j = decltype(jc)::value;
     const unsigned char* base = smem + st;
     const unsigned char* abase = base + j * A_STEP;
     u32x4 wa = *reinterpret_cast<const u32x4*>(base + w_rd[j][0]), wb;
@@ -237,6 +259,7 @@ __global__ __launch_bounds__(64 * NW * KH) void dma_kernel(const StreamParams p)
       constexpr int i = r / RPB, sub = r % RPB;
       constexpr int pb = r & 1;  // partial set of this run
       constexpr int ab = i & 1;  // fragment set of this block
+      issue_slot(ic<j * NRUN + r>{}, i_next, t_next);
       if (sub == 0 && i + 1 < MB) {
 #pragma unroll
         for (int t = 0; t < 4; t++) Af[ab ^ 1][t] = *reinterpret_cast<const h8*>(abase + a_rd[t] + (i + 1) * 4096);
@@ -266,10 +289,11 @@ __global__ __launch_bounds__(64 * NW * KH) void dma_kernel(const StreamParams p)
       if (i < upp) {
         wait_vm<(D - 2) * L>();
         wg_barrier();
-        issue(i + D - 1, (t + D - 1) % D);
         if (i < my_units) {
-          step(part * PART + t * STAGE, 0);
-          step(part * PART + t * STAGE, 1);
+          step(part * PART + t * STAGE, ic<0>{}, i + D - 1, (t + D - 1) % D);
+          step(part * PART + t * STAGE, ic<1>{}, i + D - 1, (t + D - 1) % D);
+        } else {
+          issue(i + D - 1, (t + D - 1) % D);  // a part that has run out of units keeps the count of its queue
         }
       }
     });
@@ -322,7 +346,6 @@ struct Shape {
 
 // By rows unless the knob names one (any shape runs any M; a row's bits depend on the shape, not on M)
 Shape shape_of(const MatmulArgs& a, const Tune& t) {
-  if (t.skinny_shape == 1) return Shape{1, 4, 4, 2};
   if (t.skinny_shape == 2) return Shape{2, 4, 2, 3};
   if (t.skinny_shape == 3) return Shape{1, 2, 4, 3};
   return a.M <= 32 ? Shape{1, 2, 4, 3} : Shape{2, 4, 2, 3};
@@ -333,6 +356,7 @@ hipError_t launch_shape(const StreamParams& p, hipStream_t s) {
   constexpr int ROWS = MB * 32;
   constexpr size_t smem = (size_t)KH * D * (2 * ROWS * 128 + NW * 32 * 64 + NW * 256);
   static_assert(smem <= 160 * 1024, "LDS of a CU");
+  static_assert(64 * NW * KH <= 1024, "threads of a workgroup");
   auto go = [&](auto k) {
     if (smem > 64 * 1024) (void)hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     hipLaunchKernelGGL(k, dim3(p.mtiles * p.ngroups * p.ksplit), dim3(64 * NW * KH), smem, s, p);
@@ -344,8 +368,7 @@ hipError_t launch_shape(const StreamParams& p, hipStream_t s) {
 
 template <bool AFFINE>
 hipError_t launch_affine(const StreamParams& p, const Shape& sh, hipStream_t s) {
-  if (sh.mb == 1 && sh.nw == 2) return launch_shape<1, 2, 4, 3, AFFINE>(p, s);
-  if (sh.mb == 1) return launch_shape<1, 4, 4, 2, AFFINE>(p, s);
+  if (sh.mb == 1) return launch_shape<1, 2, 4, 3, AFFINE>(p, s);
   return launch_shape<2, 4, 2, 3, AFFINE>(p, s);
 }
 
@@ -379,6 +402,7 @@ uint32_t skinny_dma_ksplit(const MatmulArgs& a, const Tune& t) {
   while (want > 1 && (want - 1) * ((nunits + want - 1) / want) >= nunits) want--;
   return want;
 }
+
 
 hipError_t launch_skinny_dma(StreamParams& p, const MatmulArgs& a, const Tune& t, hipStream_t s) {
   const Shape sh = shape_of(a, t);
