@@ -31,9 +31,16 @@
 namespace ztvm {
 namespace {
 
-// 4 bytes per lane: global (base + voff) -> LDS (lds_base + 4*lane)
-__device__ __forceinline__ void dma4(const void* base, uint32_t voff, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" : : "v"(voff), "s"(base), "s"(lds_base) : "memory", "m0");
+
+// Transfers global (base + voff) -> LDS (lds_base + 16*lane, or + 4*lane). Not a memory barrier for the compiler, so
+// that it may move the LDS reads of the next run of matrix instructions above a transfer: the order that matters (a
+// stage is refilled only after the barrier that follows its last read, and read only after the wait and the barrier
+// that follow its transfers) is kept by the wait and barrier statements, which are.
+__device__ __forceinline__ void xfer16(const void* base, uint32_t voff, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(base), "s"(lds_base));
+}
+__device__ __forceinline__ void xfer4(const void* base, uint32_t voff, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" : : "v"(voff), "s"(base), "s"(lds_base));
 }
 
 // weight rows of 64 bytes: a 128-bit read serves 8 lanes a cycle, rows of equal parity share a bank half
@@ -51,7 +58,6 @@ __global__ __launch_bounds__(64 * NW * KH) void dma_kernel(const StreamParams p)
   constexpr int L = 2 * AP + 2 + 1;      // transfers per wave and unit
   static_assert(ROWS * 8 % T == 0, "whole pieces per thread");
   static_assert(D >= 2 && (D - 1) * L < 64, "the queue counter holds 63");
-  static_assert((KH - 1) * NW * MB * 4096 <= KH * PART, "the parts' totals fit the pipeline's LDS");
 
   extern __shared__ __align__(16) unsigned char smem[];
   const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_ptr_t)smem;
@@ -84,7 +90,7 @@ __global__ __launch_bounds__(64 * NW * KH) void dma_kernel(const StreamParams p)
   const uint32_t u_last = u_stop - 1;  // fetches past the part's share repeat the split's last unit; nobody reads them
 
   // ---- transfers. Piece q = r*T + tp of a step's activation tile is LDS bytes [16q, 16q+16): row q/8, chunk slot q%8.
-  uint32_t a_off[AP];
+  uint32_t a_off[AP], xs_off[AP];  // activations; their group sums (the bias term's left operand)
 #pragma unroll
   for (int r = 0; r < AP; r++) {
     const uint32_t q = r * T + tp, row = q >> 3;
@@ -92,6 +98,7 @@ __global__ __launch_bounds__(64 * NW * KH) void dma_kernel(const StreamParams p)
     uint32_t m = m0 + row;
     if (CLAMP) m = m < p.M ? m : p.M - 1;
     a_off[r] = (m * p.K + ch * 8) * 2u;
+    xs_off[r] = (m * p.xs_stride + ch * 8) * 2u;
   }
   // Piece q = r*T + tp (r = 0, 1) of a unit's weight tile: row q/4, chunk slot q%4.
   uint32_t w_off[2];
@@ -107,6 +114,9 @@ __global__ __launch_bounds__(64 * NW * KH) void dma_kernel(const StreamParams p)
   ncol = ncol < p.N ? ncol : p.N - 1;
   const uint32_t s_off = (ncol * p.spr + (AFFINE ? 0u : 2u * h)) * 2u;
   const uint32_t lds_part = lds0 + part * PART;
+  const bool with_bias = AFFINE && split == 0;
+  // bias step of this part that travels as step j of the unit sent e turns past the end (see the bias term below)
+  auto bias_step_of = [&](uint32_t e, int j) __attribute__((always_inline)) { return (2 * e + j) * KH + part; };
   // Transfer k (0 .. L-1) of unit i of this part's sequence, into stage t: the activations of step 0, of step 1, the
   // weights, the scales.
   auto issue_one = [&](auto kc, uint32_t i, uint32_t t) __attribute__((always_inline)) {
@@ -116,12 +126,16 @@ __global__ __launch_bounds__(64 * NW * KH) void dma_kernel(const StreamParams p)
     const uint32_t st = lds_part + t * STAGE;
     if constexpr (k < 2 * AP) {
       constexpr int j = k / AP, r = k % AP;
-      dma16<0>(reinterpret_cast<const char*>(p.inp) + (size_t)u * 256 + j * 128, a_off[r], st + j * A_STEP + (r * NW + wc) * 1024u);
+      const uint32_t bs = bias_step_of(i - upp, j);  // only meant for i >= upp
+      if (with_bias && i >= upp && bs < p.bias_steps)
+        xfer16(p.xs16 + bs * KS, xs_off[r], st + j * A_STEP + (r * NW + wc) * 1024u);
+      else
+        xfer16(reinterpret_cast<const char*>(p.inp) + (size_t)u * 256 + j * 128, a_off[r], st + j * A_STEP + (r * NW + wc) * 1024u);
     } else if constexpr (k < 2 * AP + 2) {
       constexpr int r = k - 2 * AP;
-      dma16<0>(reinterpret_cast<const char*>(p.weights) + (size_t)u * 64, w_off[r], st + A_BYTES + (r * NW + wc) * 1024u);
+      xfer16(reinterpret_cast<const char*>(p.weights) + (size_t)u * 64, w_off[r], st + A_BYTES + (r * NW + wc) * 1024u);
     } else {
-      dma4(reinterpret_cast<const char*>(p.scales) + (size_t)u * (AFFINE ? 4 : 8), s_off, st + A_BYTES + W_BYTES + wc * 256u);
+      xfer4(reinterpret_cast<const char*>(p.scales) + (size_t)u * (AFFINE ? 4 : 8), s_off, st + A_BYTES + W_BYTES + wc * 256u);
     }
   };
   // transfers [L*slot/NSLOT, L*(slot+1)/NSLOT): a turn sends its L transfers in NSLOT helpings, between its runs of
@@ -163,55 +177,38 @@ __global__ __launch_bounds__(64 * NW * KH) void dma_kernel(const StreamParams p)
     for (int e = 0; e < 16; e++) tot[i][e] = 0.f;
   const f16v zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 
-  // ---- the pipeline's first D-1 units go out before anything else
+  // ---- the pipeline's first D-1 units go out before anything else. (All workgroups of the chip start at the same
+  // moment on cold caches: the first barrier comes 9000 ticks into a 48000-tick kernel at 128 rows. Sending one unit
+  // and the next after the first barrier only puts two such trips one after the other.)
 #pragma unroll
   for (int t = 0; t < D - 1; t++) issue(t, t);
 
-  // ---- bias term (affine, first k split, k part 0): tot = [xs_hi | xs_lo] x biases, 64 columns per step; the group
-  // sums go through stage D-1 of part 0, which the pipeline first fills after the first barrier of its loop.
-  if (AFFINE && split == 0) {
+  // ---- bias term (affine, first k split): tot += [xs_hi | xs_lo] x biases, 64 columns per step, after the main loop.
+  // Bias step (2e + j)*KH + part belongs to this part: its group sums travel as the "activations" of step j of the
+  // unit that the pipeline sends e turns past its end (it sends D-1 units past the end anyway, to keep the count of
+  // its queue), so they are in LDS when the loop ends; the biases of e = 0, j = 0 wait in registers from here on. Fetched
+  // and multiplied before the loop, the term kept every wave waiting for one more trip to memory at the start.
+  auto load_biases = [&](uint32_t bs, h8* dst) __attribute__((always_inline)) {
     const uint32_t G = p.spr;
     const _Float16* brow = p.biases + (size_t)ncol * G;
-    const uint32_t bst = (D - 1) * STAGE;  // part 0
-    for (uint32_t bs = 0; bs < p.bias_steps; bs++) {
-      h8 bf[4];
-      if (part == 0) {
 #pragma unroll
-        for (int r = 0; r < AP; r++) {
-          const uint32_t q = r * T + tp, row = q >> 3;
-          const uint32_t ch = (q & 7u) ^ swz(row);
-          uint32_t m = m0 + row;
-          if (CLAMP) m = m < p.M ? m : p.M - 1;
-          dma16<0>(p.xs16 + bs * KS, (m * p.xs_stride + ch * 8) * 2u, lds0 + bst + (r * NW + wc) * 1024u);
+    for (int t = 0; t < 4; t++) {
+      const uint32_t col = bs * KS + chunk_of(t) * 8;  // column c of [hi | lo] meets b[n][c mod G]; zero past 2G
+      h8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (bs < p.bias_steps && col < 2 * G) {
+        if (G % 8 == 0) {
+          v = *reinterpret_cast<const h8*>(brow + (col % G));
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; e++)
+            if (col + e < 2 * G) v[e] = brow[(col + e) % G];
         }
-#pragma unroll
-        for (int t = 0; t < 4; t++) {
-          const uint32_t col = bs * KS + chunk_of(t) * 8;
-          h8 v = {0, 0, 0, 0, 0, 0, 0, 0};
-          if (col < 2 * G) {
-            if (G % 8 == 0) {
-              v = *reinterpret_cast<const h8*>(brow + (col % G));
-            } else {
-#pragma unroll
-              for (int e = 0; e < 8; e++)
-                if (col + e < 2 * G) v[e] = brow[(col + e) % G];
-            }
-          }
-          bf[t] = v;
-        }
-        wait_vm<0>();
       }
-      wg_barrier();
-      if (part == 0) {
-#pragma unroll
-        for (int i = 0; i < MB; i++)
-#pragma unroll
-          for (int t = 0; t < 4; t++)
-            tot[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const h8*>(smem + bst + a_rd[t] + i * 4096), bf[t], tot[i], 0, 0, 0);
-      }
-      wg_barrier();
+      dst[t] = v;
     }
-  }
+  };
+  h8 bf0[4];  // the biases of this part's bias step e = 0, j = 0, in registers from here to the end of the loop
+  if (with_bias) load_biases(bias_step_of(0, 0), bf0);
 
   // ---- main loop
   h8 Af[2][4], Bf[4];
@@ -302,9 +299,35 @@ __global__ __launch_bounds__(64 * NW * KH) void dma_kernel(const StreamParams p)
 #pragma unroll
   for (int e = 0; e < 16; e++) tot[MB - 1][e] = __builtin_fmaf(sc_prev, acc[1][e], tot[MB - 1][e]);
 
+  wait_vm<0>();  // the units sent past the end have landed (their weights and scales: nobody reads them)
+  wg_barrier();
+  if (with_bias) {
+    for (uint32_t e = 0; e < D - 1; e++) {
+      const uint32_t st = part * PART + ((upp + e) % D) * STAGE;
+#pragma unroll
+      for (int j = 0; j < 2; j++) {
+        if (bias_step_of(e, j) < p.bias_steps) {  // uniform per wave
+          h8 bf[4];
+          if (e == 0 && j == 0) {
+#pragma unroll
+            for (int t = 0; t < 4; t++) bf[t] = bf0[t];
+          } else {
+            load_biases(bias_step_of(e, j), bf);  // more than KH bias steps (K above 2048*KH): fetched now
+          }
+#pragma unroll
+          for (int i = 0; i < MB; i++)
+#pragma unroll
+            for (int t = 0; t < 4; t++)
+              tot[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const h8*>(smem + st + j * A_STEP + a_rd[t] + i * 4096), bf[t], tot[i], 0, 0,
+                                                              0);
+        }
+      }
+    }
+  }
+
   // ---- the k parts add up through LDS, in part order
+  constexpr uint32_t RED_BYTES = (KH - 1) * NW * MB * 4096;
   if (KH > 1) {
-    wait_vm<0>();  // the fetches past the end still write LDS
     wg_barrier();
     float* red = reinterpret_cast<float*>(smem);
     if (part > 0) {
@@ -314,17 +337,43 @@ __global__ __launch_bounds__(64 * NW * KH) void dma_kernel(const StreamParams p)
         for (int e = 0; e < 16; e++) red[(((part - 1) * NW + wc) * MB + i) * 1024 + e * 64 + lane] = tot[i][e];
     }
     wg_barrier();
-    if (part > 0) return;
-    for (uint32_t pp = 1; pp < KH; pp++)
+    if (part == 0) {
+      for (uint32_t pp = 1; pp < KH; pp++)
+#pragma unroll
+        for (int i = 0; i < MB; i++)
+#pragma unroll
+          for (int e = 0; e < 16; e++) tot[i][e] += red[(((pp - 1) * NW + wc) * MB + i) * 1024 + e * 64 + lane];
+    }
+  }
+
+  // ---- f16 results of a whole k range leave as full rows of the workgroup's tile: through LDS (behind the parts'
+  // totals, which part 0 may still be reading), 16 bytes per lane, every wave of the workgroup storing. Stored from
+  // the accumulator layout a lane writes 2 bytes and an instruction 64 bytes of each of two rows: 3 us of a 29 us
+  // kernel at 128 rows.
+  // D layout of a 32x32 block: lane -> column frow, register e -> row 8*(e/4) + 4*h + e%4
+  if (p.ksplit == 1 && !p.out_f32 && p.N % 8 == 0 && (reinterpret_cast<uintptr_t>(p.out) & 15u) == 0) {
+    constexpr uint32_t PITCH = CW * 2 + 16;  // the two rows an instruction writes fall into different banks
+    static_assert(RED_BYTES + ROWS * PITCH <= KH * PART, "the output tile fits behind the totals");
+    unsigned char* ot = smem + RED_BYTES;
+    if (part == 0) {
 #pragma unroll
       for (int i = 0; i < MB; i++)
 #pragma unroll
-        for (int e = 0; e < 16; e++) tot[i][e] += red[(((pp - 1) * NW + wc) * MB + i) * 1024 + e * 64 + lane];
-  } else {
-    wait_vm<0>();
+        for (int e = 0; e < 16; e++) {
+          const uint32_t row = i * 32 + 8 * (e / 4) + 4 * h + (e % 4);
+          *reinterpret_cast<_Float16*>(ot + row * PITCH + (wc * 32 + frow) * 2) = (_Float16)tot[i][e];
+        }
+    }
+    wg_barrier();
+    for (uint32_t q = tid; q < ROWS * CW / 8; q += 64 * NW * KH) {
+      const uint32_t row = q / (CW / 8), c8 = q % (CW / 8);
+      const uint32_t m = m0 + row, n = n0 + c8 * 8;
+      if (m < p.M && n < p.N)
+        *reinterpret_cast<u32x4*>(reinterpret_cast<_Float16*>(p.out) + (size_t)m * p.N + n) = *reinterpret_cast<const u32x4*>(ot + row * PITCH + c8 * 16);
+    }
+    return;
   }
-
-  // D layout of a 32x32 block: lane -> column frow, register e -> row 8*(e/4) + 4*h + e%4
+  if (part > 0) return;
   const uint32_t nn = n0 + wc * 32 + frow;
 #pragma unroll
   for (int i = 0; i < MB; i++)
@@ -377,6 +426,7 @@ hipError_t launch_affine(const StreamParams& p, const Shape& sh, hipStream_t s) 
 bool skinny_dma_supports(const MatmulArgs& a, const Tune& t) {
   if (t.skinny_dma == 1) return false;  // switched off
   if (a.bits != 4 || a.slots != 0 || a.M < 2 || a.K % 128 != 0) return false;
+  if (a.affine && 2 * a.spr > 8 * 64) return false;  // the bias term's steps ride on the units sent past the end: at most 2*KH*(D-1)
   const uint64_t lim = 1ull << 32;
   return (uint64_t)a.N * a.k_packed * 4 < lim && (uint64_t)a.N * a.spr * 2 < lim && (uint64_t)a.M * a.K * 2 < lim &&
          (uint64_t)a.M * (2 * a.spr + 64) * 2 < lim;  // the last: rows of group sums, at most 2*spr + 63 wide
@@ -402,6 +452,7 @@ uint32_t skinny_dma_ksplit(const MatmulArgs& a, const Tune& t) {
   while (want > 1 && (want - 1) * ((nunits + want - 1) / want) >= nunits) want--;
   return want;
 }
+
 
 
 hipError_t launch_skinny_dma(StreamParams& p, const MatmulArgs& a, const Tune& t, hipStream_t s) {
