@@ -33,7 +33,7 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 # HBM bytes per GEMV launch (mean of the three configs[1] shapes) from two `rocprofv3 --pmc` runs of
 # `bench.py --pmc` (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from a 256 MiB copy);
 # summary in profiles/gemv_int4_configs1_hbm_traffic.md
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = 26.96e6
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 27.00e6
 ROTATION_FLOOR_BYTES = 300e6   # distinct operand bytes a memory-bound row rotates over: past the 256 MB last-level cache
 ROUNDS = 5                     # timed replays of the headline; the median is reported
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense f16 MFMA, published
@@ -182,7 +182,8 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the per-shape, GEMM, MoE and int3 extras")
     ap.add_argument("--pmc", action="store_true",
                     help="counter-collection mode for `rocprofv3 --pmc`: a few eager launches of a 256 MiB copy "
-                         "(calibration), of each configs[1] GEMV and of the M=512 prefill GEMM, no timing")
+                         "(calibration), of each configs[1] GEMV, of the M=512 prefill GEMM and of the small-batch "
+                         "families (M = 8, 32, 128), no timing")
     ap.add_argument("--option", action="append", default=[], help="name=value launch knob (ztvm_set_option)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -216,6 +217,11 @@ def main():
                   for r in range(2)]
         for r in range(6):
             ctx.matmul(gdescs[r % 2])
+        # the small-batch families at their bench shapes (family chosen by the library), six launches each over two sets
+        for bits, M in ((4, 8), (3, 8), (4, 32), (4, 128), (8, 128)):
+            bdescs = [make_desc(capi, bits, K, N, M, upload_set(ctx, synth, K, N, bits, salt=r, M=M)[0]) for r in range(2)]
+            for r in range(6):
+                ctx.matmul(bdescs[r % 2])
         ctx.sync()
         ctx.close()
         print(json.dumps({"pmc_mode": True, "copy_bytes": nbytes}))

@@ -578,8 +578,35 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
     for (int e = 0; e < 16; e++) tot[1][j][e] = __builtin_fmaf(sc[SCALES - 1][j], part[1][j][e], tot[1][j][e]);
 
   // D layout of a 32x32 block: lane -> column n = lane % 32, register e -> row 8*(e/4) + 4*(lane/32) + e%4.
-  // The lane's part of the store addresses is computed here, not carried through the loop.
+  // Tile rows come in the groups of eight the activations were fetched in; a group moved back writes the values the
+  // group before it writes, to the same places.
   const uint32_t ln = opaque(lane);
+  const uint32_t last = p.M >= 8 ? p.M - 8 : 0;
+  if (p.N % 8 == 0 && (reinterpret_cast<uintptr_t>(p.out) & 15u) == 0) {
+    // The tile leaves as full rows: through LDS (the stages are done with), 16 bytes per lane. Stored from the
+    // accumulator layout a lane writes 2 bytes and an instruction 64 bytes of each of two rows.
+    constexpr uint32_t PITCH = TN * 2 + 16;  // the two rows an instruction writes fall into different banks
+    static_assert((size_t)TM * PITCH <= NSTAGE * (size_t)STAGE_BYTES, "the output tile fits the stages");
+    __builtin_amdgcn_s_waitcnt(0x0070);
+    __syncthreads();  // every wave has read its last fragments
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+      for (int j = 0; j < 2; j++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+          const uint32_t row = wm * 64 + i * 32 + 8 * (e / 4) + 4 * (ln >> 5) + (e % 4);
+          *reinterpret_cast<_Float16*>(smem + row * PITCH + (wn * 64 + j * 32 + (ln & 31u)) * 2) = (_Float16)tot[i][j][e];
+        }
+    __syncthreads();
+    for (uint32_t q = tid; q < TM * TN / 8; q += THREADS) {
+      const uint32_t row = q / (TN / 8), c8 = q % (TN / 8);
+      const uint32_t row0 = m0 + (row & ~7u), m = (row0 < last ? row0 : last) + (row & 7u), n = n0 + c8 * 8;
+      if (row0 < p.M && m < p.M && n < p.N)
+        *reinterpret_cast<u32x4*>(p.out + (size_t)m * p.N + n) = *reinterpret_cast<const u32x4*>(smem + row * PITCH + c8 * 16);
+    }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < 2; i++)
 #pragma unroll
@@ -587,9 +614,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
       const uint32_t n = n0 + wn * 64 + j * 32 + (ln & 31u);
 #pragma unroll
       for (int e = 0; e < 16; e++) {
-        // tile rows come in the groups of eight the activations were fetched in; a group moved
-        // back writes the values the group before it writes, to the same places
-        const uint32_t row0 = m0 + wm * 64 + i * 32 + 8 * (e / 4), last = p.M >= 8 ? p.M - 8 : 0;
+        const uint32_t row0 = m0 + wm * 64 + i * 32 + 8 * (e / 4);
         const uint32_t m = (row0 < last ? row0 : last) + 4 * (ln >> 5) + (e % 4);
         if (row0 < p.M && m < p.M && n < p.N) p.out[(size_t)m * p.N + n] = (_Float16)tot[i][j][e];
       }
