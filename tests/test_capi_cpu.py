@@ -92,10 +92,13 @@ def test_explicit_kernel_that_cannot_run_is_an_error(capi):
 
 
 def test_auto_picks_a_family_by_rows(capi):
-    """M = 1: per-row GEMV; 2..16: row-group GEMV; 17..128: weight-streaming matrix-core kernel; above: tile GEMM."""
-    for M, want in ((1, capi.KERNEL_GEMV), (2, capi.KERNEL_ROWS), (16, capi.KERNEL_ROWS), (17, capi.KERNEL_SKINNY),
-                    (128, capi.KERNEL_SKINNY), (129, capi.KERNEL_GEMM)):
+    """M = 1: per-row GEMV; 2..12: row-group GEMV (to 16 for what the transfer-engine skinny kernel does not take: 3-bit,
+    8-bit, K not a multiple of 128); then to 128: weight-streaming matrix-core kernel; above: tile GEMM."""
+    for M, want in ((1, capi.KERNEL_GEMV), (2, capi.KERNEL_ROWS), (12, capi.KERNEL_ROWS), (13, capi.KERNEL_SKINNY),
+                    (17, capi.KERNEL_SKINNY), (128, capi.KERNEL_SKINNY), (129, capi.KERNEL_GEMM)):
         assert capi.resolve(good(capi, M=M)) == want, M
+    assert capi.resolve(good(capi, M=16, bits=3, k_packed=384, scales_per_row=64)) == capi.KERNEL_ROWS
+    assert capi.resolve(good(capi, M=16, k_packed=24, scales_per_row=3)) == capi.KERNEL_ROWS  # K = 192
     assert capi.resolve(good(capi, M=8, bits=3, k_packed=384, scales_per_row=64)) == capi.KERNEL_ROWS
     assert capi.resolve(good(capi, M=300, bits=3, k_packed=384, scales_per_row=64)) == capi.KERNEL_GEMM
     assert capi.resolve(good(capi, M=300, bits=3, k_packed=384, scales_per_row=64, out_f32=1)) == capi.KERNEL_SKINNY
