@@ -87,6 +87,43 @@ def test_k_split(ctx, capi, synth, oracle, bits, affine, ksplit):
     assert rel_err(got32.view(np.float32).astype(np.float64), ref, 1.0) < (4e-5 if bits == 8 else 1e-5)
 
 
+@pytest.mark.parametrize("affine", [True, False])
+@pytest.mark.parametrize("M,N,K,shape", [(24, 136, 14336, 0), (100, 136, 14336, 0), (40, 132, 1024, 0), (40, 130, 1024, 0),
+                                         (70, 264, 4096, 3), (20, 264, 4096, 2), (9, 72, 16384, 0), (9, 72, 18432, 0)])
+def test_transfer_kernel_corners(ctx, capi, synth, oracle, M, N, K, shape, affine):
+    """The 4-bit transfer-engine kernel away from the bench shape: long rows (K = 14336: seven bias steps, so some
+    ride on the second unit sent past the end and their biases are fetched after the loop; 16384 is the longest it
+    takes, 18432 goes to the register-path kernel), N that is no multiple of 8 (results leave in the accumulator
+    layout) or of 4 (no split over workgroups), either tile shape at any M, and an output that starts 2 bytes off a
+    16-byte boundary."""
+    A, w, s, b = make(synth, 4, affine, M, N, K)
+    ref = oracle.gemm(oracle.MODE_FORMULA_F64, 4, affine, M, N, K, A, w, s, b, threads=8)
+    X, W, S = ctx.alloc(A.nbytes), ctx.alloc(w.nbytes), ctx.alloc(s.nbytes)
+    B = ctx.alloc(b.nbytes) if affine else 0
+    out = ctx.alloc(M * N * 2 + 16)
+    ctx.set_option("skinny.shape", shape)
+    try:
+        got = run(ctx, capi, 4, affine, M, M, N, K, A, w, s, b, capi.KERNEL_SKINNY)
+        got32 = run(ctx, capi, 4, affine, M, M, N, K, A, w, s, b, capi.KERNEL_SKINNY, out_f32=1)
+        # the same dispatch into an output 2 bytes past a 16-byte boundary
+        ctx.upload(X, A); ctx.upload(W, w); ctx.upload(S, s)
+        if affine:
+            ctx.upload(B, b)
+        ctx.fill(out, 0, M * N * 2 + 16)
+        ctx.matmul(capi.MatmulDesc(bits=4, affine=int(affine), kernel=capi.KERNEL_SKINNY, M=M, N=N, k_packed=K // 8,
+                                   scales_per_row=K // (64 if affine else 32), out=out + 2, in_=X, scales=S, weights=W, biases=B))
+        raw = ctx.download(out, M * N * 2 + 16, np.uint16)
+    finally:
+        ctx.set_option("skinny.shape", 0)
+        for a in (X, W, S, out) + ((B,) if affine else ()):
+            ctx.free(a)
+    y = got.view(np.float16).astype(np.float64)
+    assert rel_err(y, ref, 1e-2) < 1e-2
+    assert rel_err(got32.view(np.float32).astype(np.float64), ref, 1.0) < 2e-5
+    assert raw[0] == 0 and not raw[1 + M * N:].any(), "bytes around the output were written"
+    assert np.array_equal(raw[1:1 + M * N].reshape(M, N), got), "the output's alignment changed the result"
+
+
 def test_one_hot_pins_streamed_weights(ctx, capi, synth, oracle):
     """A = rows of the identity: Y[m,n] is the dequantized weight f16(fl32(q*s+b)) of W[n,k_m], bit for bit."""
     N, K = 160, 256
