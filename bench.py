@@ -347,6 +347,26 @@ def main():
             extra["gemm_M%d_K4096_N14336" % M] = {"us": round(ms * 1e3, 2), "TFLOP/s": round(tf, 1),
                                                   "mfma_f16_frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
                                                   "rotation_MB": round(ng * (g_wb + M * 4096 * 2) / 1e6, 1)}
+        # the down projection of the same prefill chunk (K=14336 -> N=4096, M=512): 32 column tiles, where the family
+        # choice goes by an estimate of both kernels; the library's choice beside the tile GEMM forced. Weights: the
+        # headline's rotating sets of this shape; one activation buffer, one output per set
+        Kd, Nd, Md = 14336, 4096, 512
+        xa = synth.activations(Md, Kd, salt=77)
+        a_dev = _put(ctx, xa)
+        dsets = shape_sets[1]
+        outs = [ctx.alloc(Md * Nd * 2) for _ in dsets]
+        x0, w0, s0, b0 = shape_hosts[1]
+        for fam_name, kern in (("auto", capi.KERNEL_AUTO), ("tile_gemm", capi.KERNEL_GEMM)):
+            descs = [capi.MatmulDesc(bits=4, affine=1, kernel=kern, M=Md, N=Nd, k_packed=Kd // 8, scales_per_row=Kd // 64, out=o,
+                                     in_=a_dev, scales=d.scales, weights=d.weights, biases=d.biases) for d, o in zip(dsets, outs)]
+            verify(ctx, oracle, capi, descs[0], (xa, w0, s0, b0), 4, Kd, Nd, Md)
+            nd_ = len(descs)
+            ms = timed_graph(ctx, [lambda d=descs[j % nd_]: ctx.matmul(d) for j in range(2 * nd_)], reps=6, warm=6) / (2 * nd_)
+            tf = 2.0 * Md * Kd * Nd / ms / 1e9
+            extra["gemm_M512_K14336_N4096_%s" % fam_name] = {
+                "us": round(ms * 1e3, 2), "TFLOP/s": round(tf, 1), "mfma_f16_frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
+                "family": {capi.KERNEL_SKINNY: "skinny", capi.KERNEL_GEMM: "gemm"}.get(capi.resolve(descs[0]), "?"),
+                "rotation_MB": round(nd_ * shape_bytes[1] / 1e6, 1)}
         # int3 decode GEMV (configs[4], M=1)
         wb = synth.weight_bytes(14336, 4096, bits=3)
         n3 = n_sets(wb)

@@ -59,7 +59,7 @@ enum {
 enum {
   ZTVM_KERNEL_AUTO = 0,
   ZTVM_KERNEL_GEMV = 1,   /* one pass per activation row; replaces int4_matmul[_sg|_tiled|_vec4|_vec4h][_affine][_q3][_moe] */
-  ZTVM_KERNEL_SKINNY = 2, /* weights streamed once through registers, default for 17 <= M <= 128 (4-bit rows with K a multiple of 128: from 13); replaces int4_matmul_batched_m4 / _batched_dyn[_affine] */
+  ZTVM_KERNEL_SKINNY = 2, /* weights streamed once through registers, default for 17 <= M <= 128 (4-bit rows with K a multiple of 128: from 13, and above 128 rows where the tile GEMM's grid of ceil(M/256) x N/128 workgroups is estimated slower); replaces int4_matmul_batched_m4 / _batched_dyn[_affine] */
   ZTVM_KERNEL_GEMM = 3,   /* MFMA tile GEMM, default for M > 128 (4-bit, 3-bit and 8-bit rows, f16 output); replaces int4_matmul_tiled_st / _sg_e1 / _sg_e5 [_affine] and int8_affine_batched at prefill M */
   ZTVM_KERNEL_ROWS = 4    /* one pass over the weights for up to 16 rows, default for 2 <= M <= 16 (4-bit rows with K a multiple of 128: to 12); replaces int4_matmul_batched_m4 and _batched_dyn[_affine] at a speculative-verify M_ROWS */
 };
@@ -182,11 +182,14 @@ ZTVM_API int ztvm_matmul(ztvm_ctx* ctx, const ztvm_matmul_desc* desc);
 
 /* ztvm_matmul for callers that cannot allocate device memory: code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc. It has no counterpart in the reference. Same
- * descriptor, same kernels and bit-identical results, but the scratch of the rows, skinny and
+ * descriptor, same kernels and bit-identical results (one exception below), but the scratch of the rows, skinny and
  * tile-GEMM families is a fixed array of ZTVM_STATIC_SCRATCH_BYTES that lives in the library's
  * device image (one copy per GPU, held until the process ends), so this call never calls hipMalloc
  * or hipFree, whatever the shape. A dispatch that needs more scratch than that is refused with
- * ZTVM_E_UNSUPPORTED and a message that says how much (ztvm_matmul takes any size). Nothing in the
+ * ZTVM_E_UNSUPPORTED and a message that says how much (ztvm_matmul takes any size); where AUTO would
+ * give a dispatch of more than 128 rows to the skinny family and its reordered copy of the
+ * activations (M x K f16) outgrows the array, the tile GEMM runs it instead (results then agree
+ * with ztvm_matmul's to the last f16 bit or two, not bit for bit). Nothing in the
  * array has to start at zero: every kernel writes what it later reads. All calls on one GPU share
  * the array, from every context and thread: two ztvm_matmul_static dispatches that overlap on one
  * GPU (different contexts or streams) race on it; dispatches on one context are ordered and safe. */

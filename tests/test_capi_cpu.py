@@ -93,9 +93,10 @@ def test_explicit_kernel_that_cannot_run_is_an_error(capi):
 
 def test_auto_picks_a_family_by_rows(capi):
     """M = 1: per-row GEMV; 2..12: row-group GEMV (to 16 for what the transfer-engine skinny kernel does not take: 3-bit,
-    8-bit, K not a multiple of 128); then to 128: weight-streaming matrix-core kernel; above: tile GEMM."""
+    8-bit, K not a multiple of 128); then to 128: weight-streaming matrix-core kernel; above: tile GEMM, or the
+    skinny kernel where the tile GEMM's tiles would leave most CUs idle (test_skinny_or_tile_gemm_above_128_rows)."""
     for M, want in ((1, capi.KERNEL_GEMV), (2, capi.KERNEL_ROWS), (12, capi.KERNEL_ROWS), (13, capi.KERNEL_SKINNY),
-                    (17, capi.KERNEL_SKINNY), (128, capi.KERNEL_SKINNY), (129, capi.KERNEL_GEMM)):
+                    (17, capi.KERNEL_SKINNY), (128, capi.KERNEL_SKINNY)):
         assert capi.resolve(good(capi, M=M)) == want, M
     assert capi.resolve(good(capi, M=16, bits=3, k_packed=384, scales_per_row=64)) == capi.KERNEL_ROWS
     assert capi.resolve(good(capi, M=16, k_packed=24, scales_per_row=3)) == capi.KERNEL_ROWS  # K = 192
@@ -108,6 +109,30 @@ def test_auto_picks_a_family_by_rows(capi):
     odd = dict(M=300, k_packed=24, scales_per_row=3)
     assert capi.resolve(good(capi, **odd)) == capi.KERNEL_SKINNY
     assert capi.validate(good(capi, kernel=capi.KERNEL_GEMM, **odd))[0] == capi.E_UNSUPPORTED
+
+
+def test_skinny_or_tile_gemm_above_128_rows(capi):
+    """Above 128 rows the 4-bit family is chosen on an estimate of both kernels' time (rounds of workgroups over 256 CUs
+    x steps x time per step). The table is the measured winner on MI355X at each point (whole dispatch, us):
+    K=4096 N=14336: M=256 skinny 53 / gemm 62, M=320 76 / 71, M=512 103 / 74; K=14336 N=4096: M=512 92 / 213,
+    M=1024 173 / 216, M=2048 372 / 258; K=4096 N=6144: M=512 52 / 66, M=768 77 / 67; K=2048 N=8192: M=512 34 / 39,
+    M=768 48 / 40; K=4096 N=4096: M=1024 57 / 67, M=2048 120 / 81."""
+    S, G = capi.KERNEL_SKINNY, capi.KERNEL_GEMM
+    table = [(4096, 14336, ((129, S), (256, S), (320, G), (512, G), (2048, G))),
+             (14336, 4096, ((512, S), (1024, S), (2048, G))),
+             (4096, 6144, ((320, S), (512, S), (768, G), (1024, G))),
+             (2048, 8192, ((512, S), (768, G), (1024, G))),
+             (4096, 4096, ((129, S), (512, S), (1024, S), (2048, G)))]
+    for K, N, rows in table:
+        for M, want in rows:
+            assert capi.resolve(good(capi, M=M, N=N, k_packed=K // 8, scales_per_row=K // 64)) == want, (K, N, M)
+    # what only the tile GEMM takes above 128 rows stays there: 3-bit and 8-bit rows, K off a multiple of 128
+    assert capi.resolve(good(capi, M=512, N=4096, bits=3, k_packed=384, scales_per_row=64)) == G
+    assert capi.resolve(good(capi, M=512, N=4096, bits=8, k_packed=1024, scales_per_row=64)) == G
+    assert capi.resolve(good(capi, M=512, N=4096, affine=0, biases=0, k_packed=520, scales_per_row=130)) == G  # K = 4160
+    # an explicit request is honoured either way
+    big = dict(M=512, N=4096, k_packed=512, scales_per_row=64)
+    assert capi.resolve(good(capi, kernel=G, **big)) == G and capi.resolve(good(capi, **big)) == S
 
 
 def test_unchecked_experts_is_an_explicit_choice(capi):

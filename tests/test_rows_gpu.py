@@ -118,7 +118,7 @@ def test_config5_int3(ctx, capi, synth, oracle, M):
 
 def test_auto_routing(capi):
     for M, want in ((1, capi.KERNEL_GEMV), (2, capi.KERNEL_ROWS), (12, capi.KERNEL_ROWS), (13, capi.KERNEL_SKINNY),
-                    (128, capi.KERNEL_SKINNY), (129, capi.KERNEL_GEMM)):
+                    (128, capi.KERNEL_SKINNY)):
         desc = capi.MatmulDesc(bits=4, affine=1, M=M, N=256, k_packed=64, scales_per_row=8, out=4096, in_=4096, scales=4096,
                                weights=4096, biases=4096)
         assert capi.resolve(desc) == want, M

@@ -157,11 +157,41 @@ def test_config5_int3_m8(ctx, capi, synth, oracle):
     assert rel_err(got.view(np.float16).astype(np.float64), ref, 1e-2) < 1e-2
 
 
+@pytest.mark.parametrize("M,N,K,affine", [(512, 4096, 14336, True), (1000, 4096, 4096, True), (200, 4096, 4096, False),
+                                          (640, 6144, 4096, True)])
+def test_many_row_tiles(ctx, capi, synth, oracle, M, N, K, affine):
+    """The shapes the library gives this family above 128 rows (few column tiles: the tile GEMM would leave CUs idle):
+    several rounds of workgroups, a last row tile that is partly empty, with and without a k split. A sample of rows
+    against the formula, and the rows past M untouched."""
+    A, w, s, b = make(synth, 4, affine, M, N, K)
+    desc_kernel = capi.KERNEL_AUTO
+    probe = capi.MatmulDesc(bits=4, affine=int(affine), M=M, N=N, k_packed=K // 8, scales_per_row=K // (64 if affine else 32),
+                            out=4096, in_=4096, scales=4096, weights=4096, biases=4096 if affine else 0)
+    assert capi.resolve(probe) == capi.KERNEL_SKINNY
+    CAP = M + 8
+    Acap = np.concatenate([A, np.zeros((8, K), A.dtype)])
+    got = run(ctx, capi, 4, affine, M, CAP, N, K, Acap, w, s, b, desc_kernel, prefill=0x5A)
+    assert (got[M:] == 0x5A5A).all(), "rows past M were written"
+    rows = np.unique(np.concatenate([np.arange(0, M, 37), [M - 1, M - 2, 63, 64, 127, 128]]))
+    rows = rows[rows < M]
+    ref = oracle.gemm(oracle.MODE_FORMULA_F64, 4, affine, len(rows), N, K, np.ascontiguousarray(A[rows]), w, s, b, threads=8)
+    y = got[rows].view(np.float16).astype(np.float64)
+    assert rel_err(y, ref, 1e-2) < 1e-2
+    # the same rows through the tile GEMM agree to the last bits of f16
+    gemm = run(ctx, capi, 4, affine, M, CAP, N, K, Acap, w, s, b, capi.KERNEL_GEMM)
+    assert rel_err(y, gemm[rows].view(np.float16).astype(np.float64), 1e-2) < 2e-3
+
+
 def test_auto_picks_skinny(capi):
-    for M, want in ((1, capi.KERNEL_GEMV), (17, capi.KERNEL_SKINNY), (128, capi.KERNEL_SKINNY), (129, capi.KERNEL_GEMM)):
+    for M, want in ((1, capi.KERNEL_GEMV), (17, capi.KERNEL_SKINNY), (128, capi.KERNEL_SKINNY)):
         desc = capi.MatmulDesc(bits=4, affine=1, M=M, N=256, k_packed=64, scales_per_row=8, out=4096, in_=4096, scales=4096,
                                weights=4096, biases=4096)
         assert capi.resolve(desc) == want, M
+    # above 128 rows: the tile GEMM where its tiles fill the CUs, this family where they would not
+    for M, N, K, want in ((512, 14336, 4096, capi.KERNEL_GEMM), (512, 4096, 14336, capi.KERNEL_SKINNY), (2048, 4096, 14336, capi.KERNEL_GEMM)):
+        desc = capi.MatmulDesc(bits=4, affine=1, M=M, N=N, k_packed=K // 8, scales_per_row=K // 64, out=4096, in_=4096, scales=4096,
+                               weights=4096, biases=4096)
+        assert capi.resolve(desc) == want, (M, N, K)
     desc = capi.MatmulDesc(bits=3, affine=1, M=300, N=256, k_packed=48, scales_per_row=8, out=4096, in_=4096, scales=4096,
                            weights=4096, biases=4096)
     assert capi.resolve(desc) == capi.KERNEL_GEMM  # 3-bit rows: the same ladder

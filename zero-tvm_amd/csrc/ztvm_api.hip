@@ -182,8 +182,8 @@ MatmulArgs to_args(const ztvm_matmul_desc* d) {
 
 // Which family runs a descriptor. Thresholds are measured crossovers on
 // MI355X: the GEMV re-reads the weights once per activation row, the skinny
-// kernel streams them once through registers for tiles of up to 128 rows, the
-// tile GEMM needs enough rows to fill its 256-row tile.
+// kernel streams them once per tile of up to 128 rows, the tile GEMM needs
+// enough tiles to fill the CUs.
 int resolve_family(const MatmulArgs& a, uint32_t want, char* why, size_t n);
 
 int resolve(const MatmulArgs& a, uint32_t want, char* why, size_t n) {
@@ -193,6 +193,35 @@ int resolve(const MatmulArgs& a, uint32_t want, char* why, size_t n) {
     return ZTVM_E_UNSUPPORTED;
   }
   return fam;
+}
+
+// Above 128 rows two families can run 4-bit rows: the tile GEMM (256 x 128 tiles from 257 rows, 128 x 128 below; no
+// k split) and the transfer-engine skinny kernel (64 x 128 tiles, k split when the tiles are few). Per flop the tile
+// GEMM is the better kernel, but it leaves CUs idle where ceil(M/256) x N/128 tiles are few or just past a multiple
+// of the CU count (N = 4096, M = 512: 64 workgroups). The choice is made on an estimate of both, in nanoseconds,
+// fitted to measurements on MI355X at K = 2048..14336, N = 4096..14336, M = 129..2048: every family runs
+// ceil(workgroups / CUs) rounds; a 64-k step costs a tile-GEMM workgroup 0.98 us (0.8 us on the smaller tile) and
+// a skinny workgroup 0.375 us; around the steps a GEMM launch spends 10 us, a skinny launch 2 us and 4 us per
+// round, and 4 us more for the reduction of a k split. The estimate reproduces the measured winner at every
+// measured point (K=4096 N=14336: skinny up to 256 rows, 53 against 62 us; K=14336 N=4096: skinny up to 1024
+// rows, 92 against 213 us at 512; K=4096 N=4096: skinny up to 1024 rows, 32 against 66 us at 512). The CU count
+// is the constant of the GPU this library is written for, so that the choice is a function of the descriptor.
+constexpr uint64_t MODEL_CUS = 256;
+uint64_t est_gemm_ns(const MatmulArgs& a) {
+  const bool big = a.M > 256;
+  const uint64_t tm = big ? 256 : 128;
+  const uint64_t tiles = ((a.M + tm - 1) / tm) * ((a.N + 127) / 128);
+  const uint64_t rounds = (tiles + MODEL_CUS - 1) / MODEL_CUS;
+  return rounds * (a.K / 64) * (big ? 980 : 800) + 10000;
+}
+uint64_t est_skinny_ns(const MatmulArgs& a) {
+  Tune t{};
+  t.num_cus = (int)MODEL_CUS;
+  const uint64_t ks = skinny_dma_ksplit(a, t);
+  const uint64_t tiles = ((a.M + 63) / 64) * (uint64_t)((a.N + 127) / 128);
+  const uint64_t rounds = (tiles * ks + MODEL_CUS - 1) / MODEL_CUS;
+  const uint64_t steps = (a.K / 64 + ks - 1) / ks;
+  return rounds * (steps * 375 + 4000) + 2000 + (ks > 1 ? 4000 : 0);
 }
 
 int resolve_family(const MatmulArgs& a, uint32_t want, char* why, size_t n) {
@@ -217,7 +246,10 @@ int resolve_family(const MatmulArgs& a, uint32_t want, char* why, size_t n) {
   // 4-bit rows that the transfer-engine skinny kernel takes: it passes the row-group GEMV at 13 rows (16.3 against
   // 16.9 us at M = 12, 16.8 against 19.5 at M = 16; K = 4096, N = 14336)
   if (ro && !(a.M > 12 && sk && skinny_dma_supports(a, Tune{}))) return ZTVM_KERNEL_ROWS;
-  if (ge && a.M > 128) return ZTVM_KERNEL_GEMM;
+  if (ge && a.M > 128) {
+    if (sk && skinny_dma_supports(a, Tune{}) && est_skinny_ns(a) < est_gemm_ns(a)) return ZTVM_KERNEL_SKINNY;
+    return ZTVM_KERNEL_GEMM;
+  }
   if (sk) return ZTVM_KERNEL_SKINNY;
   if (ge) return ZTVM_KERNEL_GEMM;
   return ZTVM_KERNEL_GEMV;
@@ -414,8 +446,13 @@ static int matmul_impl(ztvm_ctx* ctx, const ztvm_matmul_desc* desc, bool use_sta
   int rc = validate(desc, why, sizeof why, true);
   if (rc) return fail(ctx, rc, "ztvm_matmul: %s", why);
   MatmulArgs a = to_args(desc);
-  const int fam = resolve(a, desc->kernel, why, sizeof why);
+  int fam = resolve(a, desc->kernel, why, sizeof why);
   if (fam < 0) return fail(ctx, fam, "ztvm_matmul: %s", why);
+  // the skinny family works on a reordered copy of the activations in scratch; where the choice was the library's
+  // and that copy outgrows the fixed buffer, the tile GEMM (group sums only) takes the dispatch
+  if (use_static && desc->kernel == ZTVM_KERNEL_AUTO && fam == ZTVM_KERNEL_SKINNY && a.M > 128 && gemm_supports(a) &&
+      skinny_scratch_bytes(a, ctx->tune) > (size_t)ZTVM_STATIC_SCRATCH_BYTES)
+    fam = ZTVM_KERNEL_GEMM;
   switch (fam) {
     case ZTVM_KERNEL_ROWS:
     case ZTVM_KERNEL_SKINNY:
