@@ -180,10 +180,11 @@ def main():
     ap.add_argument("--sets", type=int, default=8, help="distinct weight sets rotated through (8 x 80 MB > 256 MB cache)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the per-shape, GEMM, MoE and int3 extras")
-    ap.add_argument("--pmc", action="store_true",
+    ap.add_argument("--pmc", nargs="?", const="base", default=None, choices=["base", "down"],
                     help="counter-collection mode for `rocprofv3 --pmc`: a few eager launches of a 256 MiB copy "
-                         "(calibration), of each configs[1] GEMV, of the M=512 prefill GEMM and of the small-batch "
-                         "families (M = 8, 32, 128), no timing")
+                         "(calibration), then (base) of each configs[1] GEMV, of the M=512 prefill GEMM and of the "
+                         "small-batch families (M = 8, 32, 128), or (down) of the down projection of a 512-row "
+                         "prefill chunk (K=14336, N=4096) in the family the library picks and in the tile GEMM; no timing")
     ap.add_argument("--option", action="append", default=[], help="name=value launch knob (ztvm_set_option)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -207,6 +208,16 @@ def main():
         ctx.fill(src, 1, nbytes)
         for _ in range(3):
             ctx.copy(dst, src, nbytes)
+        if args.pmc == "down":
+            K, N, M = 14336, 4096, 512
+            for kern in (capi.KERNEL_AUTO, capi.KERNEL_GEMM):
+                ddescs = [make_desc(capi, 4, K, N, M, upload_set(ctx, synth, K, N, 4, salt=r, M=M)[0], kernel=kern) for r in range(2)]
+                for r in range(6):
+                    ctx.matmul(ddescs[r % 2])
+            ctx.sync()
+            ctx.close()
+            print(json.dumps({"pmc_mode": "down", "copy_bytes": nbytes}))
+            return
         for i, (_, K, N) in enumerate(GEMV_SHAPES):
             descs = [make_desc(capi, 4, K, N, 1, upload_set(ctx, synth, K, N, 4, salt=r)[0]) for r in range(4)]
             for r in range(8):
