@@ -30,6 +30,20 @@ const put = (name) => { const b = load(name); const buf = dev.createBuffer(b.len
   dev.fill(act, 0)
   const group = dev.bg(pipe, [out, act, put('s.bin'), put('w.bin'), dev.uniformBuf(z.densePod(K, N, 4, true, CAP)), put('b.bin')])
   const desc = dev.descriptor(group)
+  // the entry point that allocates nothing gives the same bytes as the ordinary one (M = 24 rows: scratch in use)
+  {
+    const d24 = Object.assign({}, desc, { M: 24 })
+    dev.fill(out, 0)
+    dev.matmul(d24)
+    const a = Buffer.from(dev.readBuffer(out, 0, 24 * N * 2))
+    dev.fill(out, 0)
+    dev.matmulStatic(d24)
+    const b = Buffer.from(dev.readBuffer(out, 0, 24 * N * 2))
+    if (!a.equals(b)) throw new Error('matmulStatic differs from matmul')
+    const sink = dev.createBuffer(64, 'sink')
+    dev.readProbe(act, CAP * K * 2, sink)
+    dev.sync()
+  }
   const timings = dev.probeFamilies(desc, ['gemm', 'skinny', 'rows', 'gemv'], [64, 256], { warmup: 1, rounds: 2 })
   const store = z.fileTuneStore(path.join(dir, 'tune_store.json'))
   const adapter = z.deviceFingerprint(dev.info())

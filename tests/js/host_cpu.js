@@ -92,5 +92,7 @@ const good = { bits: 4, affine: 1, M: 1, N: 64, k_packed: 512, scales_per_row: 6
 assert.strictEqual(z.validate(good).code, 0)
 assert.ok(/binding 5/.test(z.validate(Object.assign({}, good, { biases: 0n })).why))
 assert.ok(/SCALES_PER_ROW/.test(z.validate(Object.assign({}, good, { scales_per_row: 63 })).why))
-assert.strictEqual(z.resolve(Object.assign({}, good, { M: 512 })), z.KERNEL.GEMM)
+// above 128 rows: the tile GEMM where its tiles fill the CUs, the skinny family where they would not
+assert.strictEqual(z.resolve(Object.assign({}, good, { M: 512, N: 14336 })), z.KERNEL.GEMM)
+assert.strictEqual(z.resolve(Object.assign({}, good, { M: 512, N: 4096 })), z.KERNEL.SKINNY)
 console.log('js host cpu checks ok')

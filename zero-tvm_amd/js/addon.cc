@@ -306,6 +306,28 @@ napi_value Matmul(napi_env env, napi_callback_info info) {  // (ctx, desc)
   return undefined(env);
 }
 
+napi_value MatmulStatic(napi_env env, napi_callback_info info) {  // (ctx, desc): ztvm_matmul that allocates nothing
+  napi_value a[2];
+  void* p;
+  ztvm_matmul_desc d;
+  if (!get_args(env, info, 2, a) || !get_ptr(env, a[0], &p) || !get_desc(env, a[1], &d)) return nullptr;
+  int rc = ztvm_matmul_static((ztvm_ctx*)p, &d);
+  if (rc) return throw_ztvm(env, (ztvm_ctx*)p, rc, "ztvm_matmul_static");
+  return undefined(env);
+}
+
+napi_value ReadProbe(napi_env env, napi_callback_info info) {  // (ctx, src, bytes, sink)
+  napi_value a[4];
+  void* p;
+  uint64_t s = 0, n = 0, k = 0;
+  if (!get_args(env, info, 4, a) || !get_ptr(env, a[0], &p) || !get_u64(env, a[1], &s) || !get_u64(env, a[2], &n) ||
+      !get_u64(env, a[3], &k))
+    return nullptr;
+  int rc = ztvm_read_probe((ztvm_ctx*)p, s, (size_t)n, k);
+  if (rc) return throw_ztvm(env, (ztvm_ctx*)p, rc, "ztvm_read_probe");
+  return undefined(env);
+}
+
 napi_value Dequant(napi_env env, napi_callback_info info) {  // (ctx, desc)
   napi_value a[2];
   void* p;
@@ -569,7 +591,7 @@ napi_value Init(napi_env env, napi_value exports) {
   static const E table[] = {
       {"abiVersion", AbiVersion}, {"create", Create}, {"destroy", Destroy}, {"deviceInfo", DeviceInfo}, {"alloc", Alloc},
       {"free", Free}, {"upload", Upload}, {"download", Download}, {"fill", Fill}, {"copy", Copy}, {"sync", Sync},
-      {"validate", Validate}, {"resolve", Resolve}, {"matmul", Matmul}, {"dequant", Dequant}, {"recordBegin", RecordBegin},
+      {"validate", Validate}, {"resolve", Resolve}, {"matmul", Matmul}, {"matmulStatic", MatmulStatic}, {"readProbe", ReadProbe}, {"dequant", Dequant}, {"recordBegin", RecordBegin},
       {"recordEnd", RecordEnd}, {"submit", Submit}, {"cmdbufDestroy", CmdbufDestroy}, {"setOption", SetOption},
       {"siluMul", SiluMul}, {"moeCombine", MoeCombine}, {"moeRouterLogits", MoeRouterLogits}, {"moeRouterTopk", MoeRouterTopk},
       {"moeSlotTranslate", MoeSlotTranslate}, {"ffnGated", FfnGated}, {"ffnGatedPrologue", FfnGatedPrologue}, {"repackPart", RepackPart},

@@ -48,6 +48,8 @@ export declare class Device {
   kvQuantizeInt8(bufs: BindEntry[], pod: Uniform, model: { kvHeads: number; headDim: number; pageSize: number },
     tokens?: number): void
   matmul(desc: MatmulDesc): void
+  matmulStatic(desc: MatmulDesc): void
+  readProbe(buffer: ZtvmBuffer, bytes: number, sink: ZtvmBuffer): void
   probeFamilies(desc: MatmulDesc, families: KernelFamily[], Ms?: number[],
     opts?: { warmup?: number; rounds?: number }): TuneTimings
   beginEncoder(): void

@@ -328,6 +328,12 @@ class Device {
 
   // one ztvm_matmul from a ready descriptor (what dispatch() builds from a pipeline and a bind group)
   matmul(desc) { addon().matmul(this.ctx, desc) }
+  // the same dispatch with the library's fixed scratch array: no device allocation, whatever the shape (for callers
+  // under graph capture or in loops that must not allocate); throws where the dispatch needs more scratch than that
+  matmulStatic(desc) { addon().matmulStatic(this.ctx, desc) }
+  // a kernel that only reads `bytes` of `buffer` (`sink`: four bytes it practically never writes): the streaming-read time
+  // of this device, to put a GEMV's time beside
+  readProbe(buffer, bytes, sink) { addon().readProbe(this.ctx, buffer.addr, bytes, sink.addr) }
 
   // Time this library's kernel families on `desc` (gemm_tune.js: probeFamilies) with this device's queue.
   probeFamilies(desc, families, Ms, opts) {
