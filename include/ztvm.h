@@ -59,7 +59,7 @@ enum {
 enum {
   ZTVM_KERNEL_AUTO = 0,
   ZTVM_KERNEL_GEMV = 1,   /* one pass per activation row; replaces int4_matmul[_sg|_tiled|_vec4|_vec4h][_affine][_q3][_moe] */
-  ZTVM_KERNEL_SKINNY = 2, /* weights streamed once through registers, default for 17 <= M <= 128 (4-bit rows with K a multiple of 128: from 13, and above 128 rows where the tile GEMM's grid of ceil(M/256) x N/128 workgroups is estimated slower); replaces int4_matmul_batched_m4 / _batched_dyn[_affine] */
+  ZTVM_KERNEL_SKINNY = 2, /* weights streamed once through registers, default for 17 <= M <= 128 (4-bit rows with K a multiple of 128: from 13), and above 128 rows where the tile GEMM's grid of ceil(M/256) x N/128 workgroups is estimated slower; replaces int4_matmul_batched_m4 / _batched_dyn[_affine] */
   ZTVM_KERNEL_GEMM = 3,   /* MFMA tile GEMM, default for M > 128 (4-bit, 3-bit and 8-bit rows, f16 output); replaces int4_matmul_tiled_st / _sg_e1 / _sg_e5 [_affine] and int8_affine_batched at prefill M */
   ZTVM_KERNEL_ROWS = 4    /* one pass over the weights for up to 16 rows, default for 2 <= M <= 16 (4-bit rows with K a multiple of 128: to 12); replaces int4_matmul_batched_m4 and _batched_dyn[_affine] at a speculative-verify M_ROWS */
 };

@@ -101,8 +101,8 @@ def test_auto_picks_a_family_by_rows(capi):
     assert capi.resolve(good(capi, M=16, bits=3, k_packed=384, scales_per_row=64)) == capi.KERNEL_ROWS
     assert capi.resolve(good(capi, M=16, k_packed=24, scales_per_row=3)) == capi.KERNEL_ROWS  # K = 192
     assert capi.resolve(good(capi, M=8, bits=3, k_packed=384, scales_per_row=64)) == capi.KERNEL_ROWS
-    assert capi.resolve(good(capi, M=300, bits=3, k_packed=384, scales_per_row=64)) == capi.KERNEL_GEMM
-    assert capi.resolve(good(capi, M=300, bits=3, k_packed=384, scales_per_row=64, out_f32=1)) == capi.KERNEL_SKINNY
+    assert capi.resolve(good(capi, M=300, N=14336, bits=3, k_packed=384, scales_per_row=64)) == capi.KERNEL_GEMM
+    assert capi.resolve(good(capi, M=300, N=14336, bits=3, k_packed=384, scales_per_row=64, out_f32=1)) == capi.KERNEL_SKINNY
     rc, why = capi.validate(good(capi, M=17, kernel=capi.KERNEL_ROWS))
     assert rc == capi.E_UNSUPPORTED and "rows" in why
     # an odd number of scales per row (K = 192) is outside the tile GEMM: the default goes to the streaming kernel
@@ -126,9 +126,16 @@ def test_skinny_or_tile_gemm_above_128_rows(capi):
     for K, N, rows in table:
         for M, want in rows:
             assert capi.resolve(good(capi, M=M, N=N, k_packed=K // 8, scales_per_row=K // 64)) == want, (K, N, M)
-    # what only the tile GEMM takes above 128 rows stays there: 3-bit and 8-bit rows, K off a multiple of 128
-    assert capi.resolve(good(capi, M=512, N=4096, bits=3, k_packed=384, scales_per_row=64)) == G
-    assert capi.resolve(good(capi, M=512, N=4096, bits=8, k_packed=1024, scales_per_row=64)) == G
+    # 3-bit and 8-bit rows and K off a multiple of 128 have the register-path skinny kernel (128-row tiles, about
+    # 1 us per step, k-split partials through memory) against the same tile GEMM. Measured, 8-bit / 3-bit:
+    # K=14336 N=4096: M=256 95 / 82 against 205 / 200, M=512 170 / 150 against 219 / 217, M=1024 325 / 282 against
+    # 223 / 220; K=4096 N=4096: M=256 47 / 44 against 64 / 63, M=512 83 / 76 against 68 / 67; K=4096 N=6144: M=256
+    # 56 / 51 against 64 / 63, M=512 101 / 92 against 69 / 67; K=4096 N=14336: M=256 91 / 81 against 66 / 63
+    for bits, kp in ((8, lambda K: K // 4), (3, lambda K: 3 * K // 32)):
+        for K, N, rows in [(14336, 4096, ((256, S), (512, S), (1024, G))), (4096, 4096, ((256, S), (512, G), (1024, G))),
+                           (4096, 6144, ((256, S), (512, G))), (4096, 14336, ((192, G), (256, G), (512, G)))]:
+            for M, want in rows:
+                assert capi.resolve(good(capi, M=M, N=N, bits=bits, k_packed=kp(K), scales_per_row=K // 64)) == want, (bits, K, N, M)
     assert capi.resolve(good(capi, M=512, N=4096, affine=0, biases=0, k_packed=520, scales_per_row=130)) == G  # K = 4160
     # an explicit request is honoured either way
     big = dict(M=512, N=4096, k_packed=512, scales_per_row=64)

@@ -137,7 +137,10 @@ def test_rules_and_routing(capi):
     ok.M = 100
     assert capi.resolve(ok) == capi.KERNEL_SKINNY        # the weight-streaming kernel up to 128 rows
     ok.M = 300
-    assert capi.resolve(ok) == capi.KERNEL_GEMM          # the tile GEMM above
+    assert capi.resolve(ok) == capi.KERNEL_SKINNY        # one column tile: the tile GEMM would run on three CUs
+    big = capi.MatmulDesc(bits=8, affine=1, M=300, N=14336, k_packed=1024, scales_per_row=64, out=4096, in_=4096, scales=4096,
+                          weights=4096, biases=4096)
+    assert capi.resolve(big) == capi.KERNEL_GEMM         # the tile GEMM above 128 rows where its tiles fill the CUs
     ok.kernel = capi.KERNEL_GEMM
     assert capi.validate(ok)[0] == 0
     ok.out_f32 = 1

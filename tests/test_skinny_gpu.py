@@ -157,29 +157,30 @@ def test_config5_int3_m8(ctx, capi, synth, oracle):
     assert rel_err(got.view(np.float16).astype(np.float64), ref, 1e-2) < 1e-2
 
 
-@pytest.mark.parametrize("M,N,K,affine", [(512, 4096, 14336, True), (1000, 4096, 4096, True), (200, 4096, 4096, False),
-                                          (640, 6144, 4096, True)])
-def test_many_row_tiles(ctx, capi, synth, oracle, M, N, K, affine):
+@pytest.mark.parametrize("M,N,K,affine,bits", [(512, 4096, 14336, True, 4), (1000, 4096, 4096, True, 4), (200, 4096, 4096, False, 4),
+                                               (640, 6144, 4096, True, 4), (512, 4096, 14336, True, 8), (250, 4096, 4096, True, 3)])
+def test_many_row_tiles(ctx, capi, synth, oracle, M, N, K, affine, bits):
     """The shapes the library gives this family above 128 rows (few column tiles: the tile GEMM would leave CUs idle):
-    several rounds of workgroups, a last row tile that is partly empty, with and without a k split. A sample of rows
-    against the formula, and the rows past M untouched."""
-    A, w, s, b = make(synth, 4, affine, M, N, K)
-    desc_kernel = capi.KERNEL_AUTO
-    probe = capi.MatmulDesc(bits=4, affine=int(affine), M=M, N=N, k_packed=K // 8, scales_per_row=K // (64 if affine else 32),
+    several rounds of workgroups, a last row tile that is partly empty, with and without a k split, in the
+    transfer-engine kernel (4-bit) and the register-path kernel (8-bit, 3-bit). A sample of rows against the formula,
+    the rows past M untouched, and agreement with the tile GEMM."""
+    A, w, s, b = make(synth, bits, affine, M, N, K)
+    probe = capi.MatmulDesc(bits=bits, affine=int(affine), M=M, N=N, k_packed=K * bits // 32, scales_per_row=K // (64 if affine else 32),
                             out=4096, in_=4096, scales=4096, weights=4096, biases=4096 if affine else 0)
     assert capi.resolve(probe) == capi.KERNEL_SKINNY
     CAP = M + 8
     Acap = np.concatenate([A, np.zeros((8, K), A.dtype)])
-    got = run(ctx, capi, 4, affine, M, CAP, N, K, Acap, w, s, b, desc_kernel, prefill=0x5A)
+    got = run(ctx, capi, bits, affine, M, CAP, N, K, Acap, w, s, b, capi.KERNEL_AUTO, prefill=0x5A)
     assert (got[M:] == 0x5A5A).all(), "rows past M were written"
     rows = np.unique(np.concatenate([np.arange(0, M, 37), [M - 1, M - 2, 63, 64, 127, 128]]))
     rows = rows[rows < M]
-    ref = oracle.gemm(oracle.MODE_FORMULA_F64, 4, affine, len(rows), N, K, np.ascontiguousarray(A[rows]), w, s, b, threads=8)
+    ref = oracle.gemm(oracle.MODE_FORMULA_F64, bits, affine, len(rows), N, K, np.ascontiguousarray(A[rows]), w, s, b, threads=8)
     y = got[rows].view(np.float16).astype(np.float64)
     assert rel_err(y, ref, 1e-2) < 1e-2
-    # the same rows through the tile GEMM agree to the last bits of f16
-    gemm = run(ctx, capi, 4, affine, M, CAP, N, K, Acap, w, s, b, capi.KERNEL_GEMM)
-    assert rel_err(y, gemm[rows].view(np.float16).astype(np.float64), 1e-2) < 2e-3
+    # the same rows through the tile GEMM agree to the last bits of f16 (byte-valued weights over a long K give
+    # outputs near 100 whose f32 sums differ more between two summation orders than near-zero outputs forgive)
+    gemm = run(ctx, capi, bits, affine, M, CAP, N, K, Acap, w, s, b, capi.KERNEL_GEMM)
+    assert rel_err(y, gemm[rows].view(np.float16).astype(np.float64), 1e-2) < (6e-3 if bits == 8 else 2e-3)
 
 
 def test_auto_picks_skinny(capi):
@@ -192,10 +193,10 @@ def test_auto_picks_skinny(capi):
         desc = capi.MatmulDesc(bits=4, affine=1, M=M, N=N, k_packed=K // 8, scales_per_row=K // 64, out=4096, in_=4096, scales=4096,
                                weights=4096, biases=4096)
         assert capi.resolve(desc) == want, (M, N, K)
-    desc = capi.MatmulDesc(bits=3, affine=1, M=300, N=256, k_packed=48, scales_per_row=8, out=4096, in_=4096, scales=4096,
+    desc = capi.MatmulDesc(bits=3, affine=1, M=300, N=14336, k_packed=384, scales_per_row=64, out=4096, in_=4096, scales=4096,
                            weights=4096, biases=4096)
     assert capi.resolve(desc) == capi.KERNEL_GEMM  # 3-bit rows: the same ladder
     for M, want in ((20, capi.KERNEL_SKINNY), (300, capi.KERNEL_GEMM)):  # 8-bit rows: the same ladder as 4-bit
-        desc = capi.MatmulDesc(bits=8, affine=1, M=M, N=256, k_packed=128, scales_per_row=8, out=4096, in_=4096, scales=4096,
+        desc = capi.MatmulDesc(bits=8, affine=1, M=M, N=14336, k_packed=1024, scales_per_row=64, out=4096, in_=4096, scales=4096,
                                weights=4096, biases=4096)
         assert capi.resolve(desc) == want, M

@@ -27,5 +27,7 @@ struct StreamParams {
 bool skinny_dma_supports(const MatmulArgs& a, const Tune& t);
 uint32_t skinny_dma_ksplit(const MatmulArgs& a, const Tune& t);
 hipError_t launch_skinny_dma(StreamParams& p, const MatmulArgs& a, const Tune& t, hipStream_t s);
+// Workgroups that share the k range of one tile in the register-path kernel (skinny.hip): a function of N and K.
+uint32_t skinny_reg_ksplit(const MatmulArgs& a, const Tune& t);
 
 }  // namespace ztvm

@@ -438,6 +438,8 @@ bool skinny_supports(const MatmulArgs& a) {
   return (uint64_t)a.M * a.K * 2 < lim && (uint64_t)a.M * (xs_stride_of(a) + 1) * 2 < lim;
 }
 
+uint32_t skinny_reg_ksplit(const MatmulArgs& a, const Tune& t) { return ksplit_of(a, t); }
+
 size_t skinny_scratch_bytes(const MatmulArgs& a, const Tune& t) {
   const uint32_t ks = skinny_dma_supports(a, t) ? skinny_dma_ksplit(a, t) : ksplit_of(a, t);
   return align256((size_t)a.M * a.K * sizeof(_Float16)) + align256((size_t)a.M * xs_stride_of(a) * sizeof(_Float16)) +

@@ -214,7 +214,24 @@ uint64_t est_gemm_ns(const MatmulArgs& a) {
   const uint64_t rounds = (tiles + MODEL_CUS - 1) / MODEL_CUS;
   return rounds * (a.K / 64) * (big ? 980 : 800) + 10000;
 }
+// The register-path skinny kernel (3-bit and 8-bit rows, K off a multiple of 128): 128-row tiles, about 1 us per
+// 64-k step, a k split that depends on N and K only and whose f32 partial results are written and read back once
+// (4 TB/s), a pre-pass that copies the activations (3 TB/s). Fitted like the others (8-bit and 3-bit, the same four
+// shapes, M = 192..1024; K=14336 N=4096 M=256: 95 against 205 us, M=512: 170 against 219; K=4096 N=4096 M=256:
+// 47 against 64).
+uint64_t est_skinny_reg_ns(const MatmulArgs& a) {
+  Tune t{};
+  t.num_cus = (int)MODEL_CUS;
+  const uint64_t ks = skinny_reg_ksplit(a, t);
+  const uint64_t tiles = ((a.M + 127) / 128) * (uint64_t)((a.N + 127) / 128);
+  const uint64_t rounds = (tiles * ks + MODEL_CUS - 1) / MODEL_CUS;
+  const uint64_t steps = (a.K / 64 + ks - 1) / ks;
+  const uint64_t partial_bytes = ks > 1 ? 2ull * a.M * a.N * 4 * ks : 0;
+  const uint64_t prep_bytes = 2ull * a.M * a.K * 2;
+  return rounds * (steps * 1000 + 4000) + 2000 + partial_bytes / 4000 + prep_bytes / 3000;
+}
 uint64_t est_skinny_ns(const MatmulArgs& a) {
+  if (!skinny_dma_supports(a, Tune{})) return est_skinny_reg_ns(a);
   Tune t{};
   t.num_cus = (int)MODEL_CUS;
   const uint64_t ks = skinny_dma_ksplit(a, t);
@@ -247,7 +264,7 @@ int resolve_family(const MatmulArgs& a, uint32_t want, char* why, size_t n) {
   // 16.9 us at M = 12, 16.8 against 19.5 at M = 16; K = 4096, N = 14336)
   if (ro && !(a.M > 12 && sk && skinny_dma_supports(a, Tune{}))) return ZTVM_KERNEL_ROWS;
   if (ge && a.M > 128) {
-    if (sk && skinny_dma_supports(a, Tune{}) && est_skinny_ns(a) < est_gemm_ns(a)) return ZTVM_KERNEL_SKINNY;
+    if (sk && est_skinny_ns(a) < est_gemm_ns(a)) return ZTVM_KERNEL_SKINNY;
     return ZTVM_KERNEL_GEMM;
   }
   if (sk) return ZTVM_KERNEL_SKINNY;
