@@ -18,7 +18,16 @@
 //     is shallow: two passes (2 KB per wave, 32 KB per CU). One pass in flight leaves the memory system idle
 //     between a wave's steps; three or more delay the activations of workgroups that start a few hundred
 //     nanoseconds later by more than they gain (measured at K=4096, N=14336: 8.5 / 7.7 / 8.9 us for 1 / 2 / 3).
-//     Only streams of dozens of rows per wave (the 248320-row LM head) pay for a third pass.
+//     Every pass in flight is three memory instructions per wave, 48 per CU, that the CU's address unit takes
+//     one after the other before any wave gets to its activations: each pass of depth costs 0.25-0.35 us of
+//     start-up (with the arithmetic taken out: 7.23 / 7.47 / 7.71 us for 1 / 2 / 3). Neither is it the
+//     first burst that costs: a third and fourth pass requested only after the activations had landed measured
+//     like the deeper ring (8.3 / 9.0 us), and so did a deeper ring whose unrolled turn no longer runs past the
+//     wave's last row (8.2 us).
+//   * the vector ALU is not the bound either: feeding the nibbles to the matrix cores as f16 subnormals (q * 2^-24:
+//     one AND per pair, no OR constant, no subtraction; 50 instead of 58 vector instructions per chunk) bought
+//     0.1 us, and is not exact: the matrix cores take subnormal operands, but a chain of them is not scale
+//     invariant (sums of products near 2^-21 lose bits below about 2^-40: 2^-18 relative per chunk).
 //   * x lives in registers: a lane always works on the same chunk index of its row part, so its 64 bytes of
 //     activations per pass are loaded from LDS once per kernel, not once per row. A wave holds at most two
 //     passes (4096 values) of a row; longer rows are shared by 2, 4 or 8 waves of the workgroup ("k parts")
@@ -202,9 +211,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_stream_kernel(const StreamGem
             part[(kpart * RG + rg) * MAX_ROWS_PER_WORKER + rr] = total;
           }
         }
+        // the wave's last row leaves the unrolled turn here (an exit, not a join: the waits of the steps before it
+        // stay as they are), so a ring deeper than a row does not run steps on rows that do not exist
+        if (U > NPW && rr + 1 >= R) goto rows_done;
       }
     }
   }
+rows_done:
 
   // ---- 5. k parts meet: part 0's wave adds the parts in part order, one row per lane ----
   if (KPARTS > 1) {
@@ -277,9 +290,9 @@ hipError_t launch_gemv_stream(const MatmulArgs& a, const Tune& t, hipStream_t s)
   uint32_t grid = (uint32_t)t.num_cus;
   const uint32_t needed = (a.N + rg - 1) / rg;
   if (grid > needed) grid = needed;
-  // passes in flight per wave: two; three where a wave streams dozens of rows and the start-up no longer matters
-  const uint32_t rows_per_worker = (a.N + grid * rg - 1) / (grid * rg);
-  const int ring = t.gemv_ring ? t.gemv_ring : (rows_per_worker >= 32 ? 3 : 2);
+  // passes in flight per wave: two, also where a wave streams dozens of rows (K=2048 N=248320: 55-61 us against
+  // 57-63 with three; K=4096 N=128256: 52.6 against 57.4)
+  const int ring = t.gemv_ring ? t.gemv_ring : 2;
   if (a.bits == 3) return launch_fmt<3, true>(p, passes, grid, ring, s);
   return a.affine ? launch_fmt<4, true>(p, passes, grid, ring, s) : launch_fmt<4, false>(p, passes, grid, ring, s);
 }
