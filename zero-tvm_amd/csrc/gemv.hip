@@ -497,7 +497,9 @@ hipError_t launch_gemv(const MatmulArgs& a, const Tune& t, hipStream_t s) {
   // (16 tokens x 8 experts, 2048 -> 512: 16.8 -> 15.4 us; 512 -> 2048: 15.5 -> 14.8 us)
   // Not down to one tile per wave: a wave with a single tile has nothing in flight behind it (4 tokens, 512 -> 2048:
   // 7.1 us on 32 workgroups of one tile per wave, 6.3 on 24 of one or two).
-  if (!t.gemv_wg_per_cu)
+  // Dense dispatches keep their grid of three workgroups per CU: a larger one no longer fits the CUs at once
+  // (8-bit, 4096 -> 14336: 13.4 us on 768 workgroups, 14.6 on 896).
+  if (!t.gemv_wg_per_cu && pairs > 1)
     for (uint32_t d = gx; d <= 2 * gx && 2 * d <= wg_tiles; d++)
       if (wg_tiles % d == 0) { gx = d; break; }
   const dim3 grid(gx, pairs, 1);
