@@ -142,6 +142,25 @@ def test_skinny_or_tile_gemm_above_128_rows(capi):
     assert capi.resolve(good(capi, kernel=G, **big)) == G and capi.resolve(good(capi, **big)) == S
 
 
+def test_family_estimate_is_sane_on_random_shapes(capi):
+    """Whatever the shape, more than 128 rows resolve to one of the two matrix-core families without an error; a grid
+    of full tiles of the tile GEMM that fills whole rounds of the 256 CUs is never given away; a single column tile is, at moderate M and K."""
+    import random
+    rnd = random.Random(7)
+    S, G = capi.KERNEL_SKINNY, capi.KERNEL_GEMM
+    for _ in range(400):
+        M = rnd.choice([129, 200, 256, 257, 400, 512, 1000, 2048, 5000, 16384])
+        K = 128 * rnd.randint(1, 256)
+        N = rnd.choice([8, 64, 120, 128, 1000, 4096, 6144, 8192, 14336, 32000, 65536])
+        fam = capi.resolve(good(capi, M=M, N=N, k_packed=K // 8, scales_per_row=K // 64))
+        assert fam in (S, G), (M, N, K, fam)
+        tiles = -(-M // 256) * -(-N // 128)
+        if M > 256 and M % 256 == 0 and tiles % 256 == 0:
+            assert fam == G, (M, N, K)
+        if N <= 128 and 1024 <= K <= 8192 and M <= 2048:   # (long rows: the skinny family's copy of the activations weighs in)
+            assert fam == S, (M, N, K)
+
+
 def test_unchecked_experts_is_an_explicit_choice(capi):
     moe = dict(N=512, k_packed=256, scales_per_row=32, slots=8, tokens=1, out_slot_stride=512, ids_stride=8, ids=0x6000)
     assert capi.validate(good(capi, **moe))[0] == capi.E_INVALID
