@@ -113,27 +113,30 @@ def test_auto_picks_a_family_by_rows(capi):
 
 def test_skinny_or_tile_gemm_above_128_rows(capi):
     """Above 128 rows the 4-bit family is chosen on an estimate of both kernels' time (rounds of workgroups over 256 CUs
-    x steps x time per step). The table is the measured winner on MI355X at each point (whole dispatch, us):
-    K=4096 N=14336: M=256 skinny 53 / gemm 62, M=320 76 / 71, M=512 103 / 74; K=14336 N=4096: M=512 92 / 213,
-    M=1024 173 / 216, M=2048 372 / 258; K=4096 N=6144: M=512 52 / 66, M=768 77 / 67; K=2048 N=8192: M=512 34 / 39,
-    M=768 48 / 40; K=4096 N=4096: M=1024 57 / 67, M=2048 120 / 81."""
+    x steps x time per step; the tile GEMM deals the tiles past its last full round to several workgroups along k).
+    The table is the measured winner on MI355X at each point (whole dispatch, us, skinny / gemm):
+    K=4096 N=14336: M=256 62 / 65, M=320 77 / 72, M=512 100 / 71, M=2048 393 / 272; K=14336 N=4096: M=512 104 / 94,
+    M=1024 172 / 143, M=2048 370 / 254; K=4096 N=6144: M=320 36 / 50, M=512 56 / 49, M=768 78 / 69, M=1024 87 / 71;
+    K=2048 N=8192: M=512 37 / 38, M=768 49 / 41, M=1024 63 / 46; K=4096 N=4096: M=256 28 / 34, M=512 34 / 44,
+    M=1024 65 / 56, M=2048 115 / 81."""
     S, G = capi.KERNEL_SKINNY, capi.KERNEL_GEMM
-    table = [(4096, 14336, ((129, S), (256, S), (320, G), (512, G), (2048, G))),
-             (14336, 4096, ((512, S), (1024, S), (2048, G))),
-             (4096, 6144, ((320, S), (512, S), (768, G), (1024, G))),
+    table = [(4096, 14336, ((129, S), (256, S), (320, G), (512, G), (640, G), (1024, G), (2048, G))),
+             (14336, 4096, ((512, G), (1024, G), (2048, G))),
+             (4096, 6144, ((320, S), (512, G), (768, G), (1024, G), (2048, G))),
              (2048, 8192, ((512, S), (768, G), (1024, G))),
-             (4096, 4096, ((129, S), (512, S), (1024, S), (2048, G)))]
+             (4096, 4096, ((129, S), (256, S), (512, S), (1024, G), (2048, G)))]
     for K, N, rows in table:
         for M, want in rows:
             assert capi.resolve(good(capi, M=M, N=N, k_packed=K // 8, scales_per_row=K // 64)) == want, (K, N, M)
     # 3-bit and 8-bit rows and K off a multiple of 128 have the register-path skinny kernel (128-row tiles, about
-    # 1 us per step, k-split partials through memory) against the same tile GEMM. Measured, 8-bit / 3-bit:
-    # K=14336 N=4096: M=256 95 / 82 against 205 / 200, M=512 170 / 150 against 219 / 217, M=1024 325 / 282 against
-    # 223 / 220; K=4096 N=4096: M=256 47 / 44 against 64 / 63, M=512 83 / 76 against 68 / 67; K=4096 N=6144: M=256
-    # 56 / 51 against 64 / 63, M=512 101 / 92 against 69 / 67; K=4096 N=14336: M=256 91 / 81 against 66 / 63
+    # 1 us per step, k-split partials through memory) against the same tile GEMM, which wins at every measured point
+    # since it splits k where its tiles are few. Measured, 8-bit / 3-bit, skinny against gemm: K=14336 N=4096: M=256
+    # 100 / 87 against 80 / 78, M=512 173 / 155 against 97 / 93, M=1024 327 / 284 against 153 / 143; K=4096 N=4096:
+    # M=256 47 / 45 against 35 / 34, M=512 81 / 77 against 45 / 44; K=4096 N=6144: M=256 56 / 52 against 45 / 44,
+    # M=512 97 / 91 against 48 / 48; K=4096 N=14336: M=256 91 / 81 against 62 / 62
     for bits, kp in ((8, lambda K: K // 4), (3, lambda K: 3 * K // 32)):
-        for K, N, rows in [(14336, 4096, ((256, S), (512, S), (1024, G))), (4096, 4096, ((256, S), (512, G), (1024, G))),
-                           (4096, 6144, ((256, S), (512, G))), (4096, 14336, ((192, G), (256, G), (512, G)))]:
+        for K, N, rows in [(14336, 4096, ((256, G), (512, G), (1024, G))), (4096, 4096, ((256, G), (512, G), (1024, G))),
+                           (4096, 6144, ((256, G), (512, G))), (4096, 14336, ((192, G), (256, G), (512, G)))]:
             for M, want in rows:
                 assert capi.resolve(good(capi, M=M, N=N, bits=bits, k_packed=kp(K), scales_per_row=K // 64)) == want, (bits, K, N, M)
     assert capi.resolve(good(capi, M=512, N=4096, affine=0, biases=0, k_packed=520, scales_per_row=130)) == G  # K = 4160

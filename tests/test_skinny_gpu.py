@@ -160,17 +160,14 @@ def test_config5_int3_m8(ctx, capi, synth, oracle):
 @pytest.mark.parametrize("M,N,K,affine,bits", [(512, 4096, 14336, True, 4), (1000, 4096, 4096, True, 4), (200, 4096, 4096, False, 4),
                                                (640, 6144, 4096, True, 4), (512, 4096, 14336, True, 8), (250, 4096, 4096, True, 3)])
 def test_many_row_tiles(ctx, capi, synth, oracle, M, N, K, affine, bits):
-    """The shapes the library gives this family above 128 rows (few column tiles: the tile GEMM would leave CUs idle):
-    several rounds of workgroups, a last row tile that is partly empty, with and without a k split, in the
-    transfer-engine kernel (4-bit) and the register-path kernel (8-bit, 3-bit). A sample of rows against the formula,
-    the rows past M untouched, and agreement with the tile GEMM."""
+    """This family above 128 rows, on shapes with few column tiles: several rounds of workgroups, a last row tile that
+    is partly empty, with and without a k split, in the transfer-engine kernel (4-bit) and the register-path kernel
+    (8-bit, 3-bit). A sample of rows against the formula, the rows past M untouched, and agreement with the tile GEMM
+    (which splits k over workgroups on these shapes)."""
     A, w, s, b = make(synth, bits, affine, M, N, K)
-    probe = capi.MatmulDesc(bits=bits, affine=int(affine), M=M, N=N, k_packed=K * bits // 32, scales_per_row=K // (64 if affine else 32),
-                            out=4096, in_=4096, scales=4096, weights=4096, biases=4096 if affine else 0)
-    assert capi.resolve(probe) == capi.KERNEL_SKINNY
     CAP = M + 8
     Acap = np.concatenate([A, np.zeros((8, K), A.dtype)])
-    got = run(ctx, capi, bits, affine, M, CAP, N, K, Acap, w, s, b, capi.KERNEL_AUTO, prefill=0x5A)
+    got = run(ctx, capi, bits, affine, M, CAP, N, K, Acap, w, s, b, capi.KERNEL_SKINNY, prefill=0x5A)
     assert (got[M:] == 0x5A5A).all(), "rows past M were written"
     rows = np.unique(np.concatenate([np.arange(0, M, 37), [M - 1, M - 2, 63, 64, 127, 128]]))
     rows = rows[rows < M]
@@ -188,8 +185,9 @@ def test_auto_picks_skinny(capi):
         desc = capi.MatmulDesc(bits=4, affine=1, M=M, N=256, k_packed=64, scales_per_row=8, out=4096, in_=4096, scales=4096,
                                weights=4096, biases=4096)
         assert capi.resolve(desc) == want, M
-    # above 128 rows: the tile GEMM where its tiles fill the CUs, this family where they would not
-    for M, N, K, want in ((512, 14336, 4096, capi.KERNEL_GEMM), (512, 4096, 14336, capi.KERNEL_SKINNY), (2048, 4096, 14336, capi.KERNEL_GEMM)):
+    # above 128 rows: the tile GEMM where its tiles (or their k parts) fill the CUs, this family where they do not
+    for M, N, K, want in ((512, 14336, 4096, capi.KERNEL_GEMM), (512, 4096, 4096, capi.KERNEL_SKINNY), (512, 4096, 14336, capi.KERNEL_GEMM),
+                          (2048, 4096, 14336, capi.KERNEL_GEMM)):
         desc = capi.MatmulDesc(bits=4, affine=1, M=M, N=N, k_packed=K // 8, scales_per_row=K // 64, out=4096, in_=4096, scales=4096,
                                weights=4096, biases=4096)
         assert capi.resolve(desc) == want, (M, N, K)

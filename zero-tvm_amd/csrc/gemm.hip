@@ -61,9 +61,12 @@ struct GemmParams {
   const uint32_t* weights;
   const _Float16* biases;
   const _Float16* xs16;  // [M][xs_stride]: hi halves, lo halves of the group sums, zero padding
+  float* partial;        // k split: [split tile][part][TM * TN] f32 totals, in the accumulators' own layout
+  uint32_t* counters;    // k split: arrivals per split tile; zero between launches
   uint32_t M, N, K, k_packed, spr;
   uint32_t mtiles, ntiles, nsteps, bias_steps, xs_stride;
   uint32_t xcd_swizzle;
+  uint32_t full_tiles, parts, steps_per_part;  // tiles [0, full_tiles) run whole; the others are dealt to `parts` workgroups
 };
 
 // LDS swizzle: a 128-bit read serves 16 lanes per cycle = two 128-byte rows of banks, and rows of
@@ -202,7 +205,7 @@ struct Seq {
   static constexpr int GRP(int p) { return AFFINE ? 0 : p / 4; }
 };
 
-template <int WM, int WN, bool AFFINE, int BITS>
+template <int WM, int WN, bool AFFINE, int BITS, bool SPLIT>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) {
   static_assert(BITS == 4 || ((BITS == 8 || BITS == 3) && AFFINE), "4-bit affine or symmetric, 8-bit and 3-bit affine");
   using S = Seq<AFFINE>;
@@ -233,11 +236,22 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
 
   // workgroup id -> tile: ids sharing an XCD (id % 8) take consecutive tiles,
   // and consecutive tiles walk m fastest, i.e. share a weight panel
-  uint32_t id = blockIdx.x;
-  const uint32_t total = p.mtiles * p.ntiles;
-  if (p.xcd_swizzle && total % 8 == 0) id = (id % 8) * (total / 8) + id / 8;
+  // Tiles past full_tiles (the last, partly filled round of workgroups, or every tile when there are few) are
+  // split along k: `parts` workgroups take consecutive step ranges of one tile and the last of them to arrive adds
+  // the parts' f32 totals in part order, so a tile's result does not depend on who arrives when.
+  // (the split tiles run as a launch of their own, SPLIT, after the whole ones)
+  uint32_t id = blockIdx.x, kpart = 0;
+  constexpr bool split = SPLIT;
+  if (SPLIT) {
+    id = p.full_tiles + blockIdx.x / p.parts;
+    kpart = blockIdx.x % p.parts;
+  } else if (p.xcd_swizzle && p.full_tiles % 8 == 0) {
+    id = (id % 8) * (p.full_tiles / 8) + id / 8;
+  }
   const uint32_t mt = id % p.mtiles, nt = id / p.mtiles;
   const uint32_t m0 = mt * TM, n0 = nt * TN;
+  const uint32_t k0 = SPLIT ? kpart * p.steps_per_part : 0;                                            // first step
+  const uint32_t nsteps = SPLIT ? (p.nsteps - k0 < p.steps_per_part ? p.nsteps - k0 : p.steps_per_part) : p.nsteps;
 
   UnpackConsts uc3;  // 3-bit: the two OR constants of the shared unpack
   if (BITS == 3) {
@@ -269,7 +283,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
   }
   const _Float16* a_base[A_LOADS];  // uniform; move one k step per fill
 #pragma unroll
-  for (int i = 0; i < A_LOADS; i++) a_base[i] = p.in + (size_t)a_row0[i] * p.K;
+  for (int i = 0; i < A_LOADS; i++) a_base[i] = p.in + (size_t)a_row0[i] * p.K + (size_t)k0 * KS;
   auto lds_slot = [&](uint32_t stage, int i) __attribute__((always_inline)) { return lds0 + stage * STAGE_BYTES + (i * WAVES + wave) * 1024u; };
 
   // ---- weights: registers, unpack, LDS
@@ -281,7 +295,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
   const uint32_t w_byte = w_n * p.k_packed * 4u + w_part * (W_CH * BITS);  // W_CH chunks of BITS bytes each
   const uint32_t w_off = w_byte & ~3u;
   // (w_byte & 3) is nonzero only for 3-bit rows with two chunks (six bytes) per thread: 2 for odd w_part
-  uint32_t w_adv = 0;  // uniform, bytes
+  uint32_t w_adv = k0 * (KS * BITS / 8);  // uniform, bytes
   uint32_t w_dst[W_CH];
 #pragma unroll
   for (int j = 0; j < W_CH; j++) w_dst[j] = W_BASE + w_row * ROW_BYTES + (((w_part * W_CH + j) ^ swz(w_row)) << 4);
@@ -342,7 +356,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
     const uint32_t sc_off = sc_n * p.spr * 2u;  // spr is even (checked on the host): rows start on 4 bytes
 #pragma unroll
     for (int k = 0; k < SC_PAIRS; k++) {
-      uint32_t e = batch * (SCB * SCALES) + 2 * k;
+      uint32_t e = k0 * SCALES + batch * (SCB * SCALES) + 2 * k;  // k0 is even: pairs stay aligned
       e = e < p.spr - 2 ? e : p.spr - 2;
       dma4(p.scales, sc_off + e * 2u, lds0 + SC_BASE + (batch & 1u) * SC_BATCH + k * (TN * 4) + wave * 256u);
     }
@@ -377,11 +391,11 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
 #pragma unroll
       for (int e = 0; e < 16; e++) tot[i][j][e] = 0.f;
   const f16v zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  f16v part_sum[2][2];  // k split: the sum of the parts, built in part order at the end
 
   // ---- the pipeline's first fetches go out before anything else: the activations of steps 0 and 1 into stages 0
   // and 1, the packed words of steps 0, 1 and 2 into registers, scale batch 0 into the ring. They land while the
   // bias term below is computed (through stage 2, which the pipeline does not touch before its first step).
-  const uint32_t nsteps = p.nsteps;
   WRegs wcur, wnext, w_first;
   if (sc_loader) load_sc(0);
   auto load_a = [&](uint32_t stage) __attribute__((always_inline)) {
@@ -401,7 +415,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
 
   // ---- bias term (affine): tot = [xs_hi | xs_lo] x biases on the matrix cores, 64 columns per step, through
   // stage 2 (two or three short steps).
-  if (AFFINE) {
+  if (AFFINE && (!SPLIT || kpart == 0)) {
     const uint32_t G = p.spr;
     const _Float16* brow = p.biases + (size_t)w_n * G;
     for (uint32_t bs = 0; bs < p.bias_steps; bs++) {
@@ -577,6 +591,58 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
 #pragma unroll
     for (int e = 0; e < 16; e++) tot[1][j][e] = __builtin_fmaf(sc[SCALES - 1][j], part[1][j][e], tot[1][j][e]);
 
+  // ---- k split: every part leaves its totals in memory (the accumulators' own layout: register r of lane l of wave
+  // w at ((w * 64 + r) * 64 + l), so every store and load is a full 256-byte run), then counts itself in; the part
+  // that finds all the others there adds the totals in part order (its own from registers, at its place in the
+  // order) and stores the tile. Nobody waits for anybody. The counter is left at zero for the next launch.
+  if constexpr (SPLIT) {
+    // The totals and the counter travel with GPU-scope accesses (written through to memory, read past the caches
+    // of this XCD), so no cache is flushed or invalidated under the workgroups that are still multiplying.
+    const uint32_t st = id - p.full_tiles;
+    uint32_t* mine = reinterpret_cast<uint32_t*>(p.partial) + ((size_t)st * p.parts + kpart) * (size_t)(TM * TN) + (size_t)wave * (64 * 64) + lane;
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+      for (int j = 0; j < 2; j++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+          const float v = tot[i][j][e];
+          __hip_atomic_store(mine + ((i * 2 + j) * 16 + e) * 64, __builtin_bit_cast(uint32_t, v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    __builtin_amdgcn_s_waitcnt(0x0070);  // every store of this wave has been acknowledged
+    __syncthreads();                     // ... and of this workgroup: only then is the arrival counted
+    volatile uint32_t* arrived = reinterpret_cast<volatile uint32_t*>(smem + SC_BASE);  // the scale ring is done with
+    if (tid == 0) *arrived = __hip_atomic_fetch_add(p.counters + st, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (*arrived != p.parts - 1) return;
+    if (tid == 0) __hip_atomic_store(p.counters + st, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    for (uint32_t q = 0; q < p.parts; q++) {
+      if (q == kpart) {  // uniform: its own totals come from the registers, at their place in the order
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+          for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) part_sum[i][j][e] = q == 0 ? tot[i][j][e] : part_sum[i][j][e] + tot[i][j][e];
+      } else {
+        const uint32_t* theirs = reinterpret_cast<const uint32_t*>(p.partial) + ((size_t)st * p.parts + q) * (size_t)(TM * TN) + (size_t)wave * (64 * 64) + lane;
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+          for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+              const float v = __builtin_bit_cast(float, __hip_atomic_load(theirs + ((i * 2 + j) * 16 + e) * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+              part_sum[i][j][e] = q == 0 ? v : part_sum[i][j][e] + v;
+            }
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+      for (int j = 0; j < 2; j++) tot[i][j] = part_sum[i][j];
+  }
+
   // D layout of a 32x32 block: lane -> column n = lane % 32, register e -> row 8*(e/4) + 4*(lane/32) + e%4.
   // Tile rows come in the groups of eight the activations were fetched in; a group moved back writes the values the
   // group before it writes, to the same places.
@@ -626,35 +692,84 @@ hipError_t launch_kernel(const GemmParams& p, hipStream_t s) {
   constexpr int TM = 64 * WM, TN = 64 * WN, THREADS = 64 * WM * WN;
   // stages + scale ring
   const size_t smem = NSTAGE * (size_t)(TM + TN) * CHUNKS * 16 + 2 * (size_t)TN * SCB * (AFFINE ? 1 : 2) * sizeof(_Float16);
-  auto k = gemm_kernel<WM, WN, AFFINE, BITS>;
-  if (smem > 64 * 1024) (void)hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-  hipLaunchKernelGGL(k, dim3(p.mtiles * p.ntiles), dim3(THREADS), smem, s, p);
+  // the whole tiles, then (a launch of their own, so that the common kernel carries nothing of the exchange) the split ones
+  if (p.full_tiles) {
+    auto k = gemm_kernel<WM, WN, AFFINE, BITS, false>;
+    if (smem > 64 * 1024) (void)hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    hipLaunchKernelGGL(k, dim3(p.full_tiles), dim3(THREADS), smem, s, p);
+  }
+  const uint32_t rest = p.mtiles * p.ntiles - p.full_tiles;
+  if (rest) {
+    auto k = gemm_kernel<WM, WN, AFFINE, BITS, true>;
+    if (smem > 64 * 1024) (void)hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    hipLaunchKernelGGL(k, dim3(rest * p.parts), dim3(THREADS), smem, s, p);
+  }
   return hipGetLastError();
 }
 
 template <int WM, int WN>
-hipError_t launch_tile(GemmParams p, bool affine, uint32_t bits, hipStream_t s) {
-  constexpr int TM = 64 * WM, TN = 64 * WN;
-  p.mtiles = (p.M + TM - 1) / TM;
-  p.ntiles = (p.N + TN - 1) / TN;
+hipError_t launch_tile(const GemmParams& p, bool affine, uint32_t bits, hipStream_t s) {
   if (bits == 8) return launch_kernel<WM, WN, true, 8>(p, s);
   if (bits == 3) return launch_kernel<WM, WN, true, 3>(p, s);
   if (affine) return launch_kernel<WM, WN, true, 4>(p, s);
   return launch_kernel<WM, WN, false, 4>(p, s);
 }
 
+// tile shape by number: rows x columns
+void tile_dims(int tile, uint32_t* tm, uint32_t* tn) {
+  *tm = tile == 3 ? 256 : (tile == 2 || tile == 4 ? 128 : 64);
+  *tn = tile == 4 ? 256 : 128;
+}
+int tile_of(const MatmulArgs& a, const Tune& t) {
+  if (t.gemm_tile >= 1 && t.gemm_tile <= 4) return t.gemm_tile;
+  return a.M > 256 ? 3 : (a.M > 64 ? 2 : 1);  // measured: 256x128 wins from M=512 up
+}
+
+uint32_t xs_stride_of(const MatmulArgs& a) { return (2 * a.spr + KS - 1) / KS * KS; }
+size_t xs_bytes_of(const MatmulArgs& a) { return a.affine ? ((size_t)a.M * xs_stride_of(a) * sizeof(_Float16) + 255) / 256 * 256 : 0; }
+
 }  // namespace
+
+// The k split of the tile GEMM. A grid of whole tiles leaves CUs idle where the tiles are few (N = 4096, M = 512:
+// 64 tiles on 256 CUs) or where the last round of workgroups is mostly empty (M = 2048, N = 14336: 896 tiles =
+// three and a half rounds). Those tiles (all of them, or the ones past the last full round) are dealt to `parts`
+// workgroups each, along k, when that fills the round: parts = CUs / tiles, at most eight, never fewer than
+// sixteen 64-k steps per part, and only where the f32 totals the parts exchange fit the scratch the caller has.
+// A function of the descriptor, the CU count and that limit: a row's bits do not depend on timing.
+GemmSplit gemm_split(const MatmulArgs& a, const Tune& t, size_t scratch_limit) {
+  uint32_t tm, tn;
+  tile_dims(tile_of(a, t), &tm, &tn);
+  const uint32_t tiles = ((a.M + tm - 1) / tm) * ((a.N + tn - 1) / tn), cus = (uint32_t)(t.num_cus > 0 ? t.num_cus : 256);
+  const uint32_t steps = a.K / KS;
+  GemmSplit g{tiles, 1, steps, 0};
+  if (t.gemm_split == 1) return g;
+  const uint32_t rest = tiles % cus;
+  if (rest == 0 || rest * 2 > cus) return g;
+  uint32_t parts = cus / rest;
+  if (parts > 8) parts = 8;
+  while (parts > 1 && steps / parts < 16) parts--;
+  if (parts < 2) return g;
+  uint32_t per = ((steps + parts - 1) / parts + 1) & ~1u;  // even: the scale pairs of a part stay 4-byte aligned
+  parts = (steps + per - 1) / per;
+  if (parts < 2 || rest > ZTVM_GEMM_SPLIT_TILES) return g;
+  const size_t bytes = (size_t)rest * parts * tm * tn * sizeof(float);
+  if (scratch_limit && xs_bytes_of(a) + bytes > scratch_limit) return g;
+  g.full_tiles = tiles - rest; g.parts = parts; g.steps_per_part = per; g.partial_bytes = bytes;
+  return g;
+}
+
 // 4-bit (affine or symmetric), 8-bit or 3-bit affine, f16 output, dense, K a multiple of 64.
 // The scales are fetched as 4-byte pairs, so a row of them must start on 4 bytes.
 bool gemm_supports(const MatmulArgs& a) {
   return a.slots == 0 && (a.bits == 4 || ((a.bits == 8 || a.bits == 3) && a.affine)) && !a.out_f32 && a.K % KS == 0 && a.spr % 2 == 0;
 }
 
-static uint32_t xs_stride_of(const MatmulArgs& a) { return (2 * a.spr + KS - 1) / KS * KS; }
+size_t gemm_scratch_bytes(const MatmulArgs& a, const Tune& t, size_t scratch_limit) {
+  return xs_bytes_of(a) + gemm_split(a, t, scratch_limit).partial_bytes;
+}
 
-size_t gemm_scratch_bytes(const MatmulArgs& a) { return a.affine ? (size_t)a.M * xs_stride_of(a) * sizeof(_Float16) : 0; }
-
-hipError_t launch_gemm(const MatmulArgs& a, const Tune& t, void* scratch, hipStream_t s) {
+// `counters`: ZTVM_GEMM_SPLIT_TILES zeroed words that belong to the caller's context (null: no k split)
+hipError_t launch_gemm(const MatmulArgs& a, const Tune& t, void* scratch, uint32_t* counters, size_t scratch_limit, hipStream_t s) {
   GemmParams p{};
   p.out = reinterpret_cast<_Float16*>(a.out);
   p.in = a.in; p.scales = a.scales; p.weights = a.weights; p.biases = a.biases;
@@ -664,14 +779,23 @@ hipError_t launch_gemm(const MatmulArgs& a, const Tune& t, void* scratch, hipStr
   p.xs_stride = xs_stride_of(a);
   p.bias_steps = a.affine ? p.xs_stride / KS : 0;
   p.xcd_swizzle = t.gemm_xcd_swizzle;
+  Tune tt = t;
+  if (!counters) tt.gemm_split = 1;
+  const GemmSplit g = gemm_split(a, tt, scratch_limit);
+  p.full_tiles = g.full_tiles; p.parts = g.parts; p.steps_per_part = g.steps_per_part;
+  p.partial = reinterpret_cast<float*>(reinterpret_cast<char*>(scratch) + xs_bytes_of(a));
+  p.counters = counters;
   if (a.affine) {
     const uint32_t pad = p.xs_stride - 2 * a.spr, cpr = a.K / 8;
     const uint32_t n = a.M * (cpr > pad ? cpr : pad);  // one thread per chunk, and enough for the padding columns
     hipLaunchKernelGGL(xsum_kernel, dim3((n + 255) / 256), dim3(256), 0, s, a.in, reinterpret_cast<_Float16*>(scratch), a.M, a.K, a.spr,
                        p.xs_stride);
   }
-  int tile = t.gemm_tile;
-  if (!tile) tile = a.M > 256 ? 3 : (a.M > 64 ? 2 : 1);  // measured: 256x128 wins from M=512 up
+  const int tile = tile_of(a, t);
+  uint32_t tm, tn;
+  tile_dims(tile, &tm, &tn);
+  p.mtiles = (a.M + tm - 1) / tm;
+  p.ntiles = (a.N + tn - 1) / tn;
   switch (tile) {
     case 3: return launch_tile<4, 2>(p, a.affine, a.bits, s);  // 256 x 128, 8 waves
     case 2: return launch_tile<2, 2>(p, a.affine, a.bits, s);  // 128 x 128, 4 waves

@@ -56,6 +56,7 @@ struct Tune {
   int rows_wg_per_cu = 0;    // the row-group GEMV: workgroups per CU and waves per workgroup (0: chosen from the LDS it stages)
   int rows_waves = 0;
   int gemm_tile = 0;        // 0 auto
+  int gemm_split = 0;       // the tile GEMM's k split: 0 = where it fills a round of workgroups, 1 = never
   int gemm_xcd_swizzle = 1;
 };
 
@@ -66,8 +67,17 @@ bool gemv_stream_supports(const MatmulArgs& a, const Tune& t);
 hipError_t launch_gemv_stream(const MatmulArgs& a, const Tune& t, hipStream_t s);
 hipError_t launch_skinny(const MatmulArgs& a, const Tune& t, void* scratch, hipStream_t s);
 size_t skinny_scratch_bytes(const MatmulArgs& a, const Tune& t);
-hipError_t launch_gemm(const MatmulArgs& a, const Tune& t, void* scratch, hipStream_t s);
-size_t gemm_scratch_bytes(const MatmulArgs& a);
+// The tile GEMM's k split for a descriptor: tiles [0, full_tiles) run whole, each of the others is dealt to `parts`
+// workgroups of steps_per_part 64-k steps, which exchange partial_bytes of f32 totals through the scratch buffer.
+struct GemmSplit {
+  uint32_t full_tiles, parts, steps_per_part;
+  size_t partial_bytes;
+};
+constexpr uint32_t ZTVM_GEMM_SPLIT_TILES = 256;  // arrival counters a context owns: at most this many split tiles
+GemmSplit gemm_split(const MatmulArgs& a, const Tune& t, size_t scratch_limit);
+// scratch_limit: the bytes the caller can give (0: as many as it takes); a split that does not fit is not made
+hipError_t launch_gemm(const MatmulArgs& a, const Tune& t, void* scratch, uint32_t* counters, size_t scratch_limit, hipStream_t s);
+size_t gemm_scratch_bytes(const MatmulArgs& a, const Tune& t, size_t scratch_limit);
 hipError_t launch_dequant(const MatmulArgs& a, hipStream_t s);
 hipError_t launch_copy(void* dst, const void* src, size_t bytes, hipStream_t s);
 hipError_t launch_read_probe(const void* src, size_t bytes, void* sink, hipStream_t s);

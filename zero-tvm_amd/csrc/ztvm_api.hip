@@ -71,6 +71,7 @@ struct ztvm_ctx {
   // context, which keep its addresses alive (scratch_pool.h).
   std::shared_ptr<DevicePool> scratch;
   void* static_scratch = nullptr;  // this device's copy of the file-scope array above
+  uint32_t* gemm_counters = nullptr;  // arrival counters of the tile GEMM's k split: zero between launches
   std::string err;
   hipDeviceProp_t prop;
 };
@@ -209,10 +210,16 @@ int resolve(const MatmulArgs& a, uint32_t want, char* why, size_t n) {
 constexpr uint64_t MODEL_CUS = 256;
 uint64_t est_gemm_ns(const MatmulArgs& a) {
   const bool big = a.M > 256;
-  const uint64_t tm = big ? 256 : 128;
-  const uint64_t tiles = ((a.M + tm - 1) / tm) * ((a.N + 127) / 128);
-  const uint64_t rounds = (tiles + MODEL_CUS - 1) / MODEL_CUS;
-  return rounds * (a.K / 64) * (big ? 980 : 800) + 10000;
+  const uint64_t step_ns = big ? 980 : 800;
+  // with the k split of the tiles past the last full round (gemm_split): the full rounds, then one round of
+  // `parts` workgroups per tile and the exchange of their f32 totals (12 us)
+  Tune t{};
+  t.num_cus = (int)MODEL_CUS;
+  const GemmSplit g = gemm_split(a, t, 0);
+  const uint64_t rounds = g.full_tiles / MODEL_CUS + (g.parts == 1 && g.full_tiles % MODEL_CUS ? 1 : 0);
+  uint64_t ns = rounds * (a.K / 64) * step_ns + 10000;
+  if (g.parts > 1) ns += g.steps_per_part * step_ns + 12000;
+  return ns;
 }
 // The register-path skinny kernel (3-bit and 8-bit rows, K off a multiple of 128): 128-row tiles, about 1 us per
 // 64-k step, a k split that depends on N and K only and whose f32 partial results are written and read back once
@@ -305,6 +312,7 @@ const Option kOptions[] = {
     {"rows.wg_per_cu", &Tune::rows_wg_per_cu},
     {"rows.waves", &Tune::rows_waves},
     {"gemm.tile", &Tune::gemm_tile},
+    {"gemm.split", &Tune::gemm_split},
     {"gemm.xcd_swizzle", &Tune::gemm_xcd_swizzle},
 };
 
@@ -322,31 +330,28 @@ int ztvm_create(int device, ztvm_ctx** out) {
   int count = 0;
   if (hipGetDeviceCount(&count) != hipSuccess || count <= 0) return fail(nullptr, ZTVM_E_NODEVICE, "no HIP device visible");
   if (device < 0 || device >= count) return fail(nullptr, ZTVM_E_INVALID, "device %d out of range (%d visible)", device, count);
-  ztvm_ctx* c = new ztvm_ctx();
+  // every exit below that is not the last one gives back what the context holds by then
+  struct Guard {
+    ztvm_ctx* c;
+    ~Guard() { if (c) ztvm_destroy(c); }
+  } g{new ztvm_ctx()};
+  ztvm_ctx* c = g.c;
   c->device = device;
   HIP_TRY(nullptr, hipSetDevice(device));
   HIP_TRY(nullptr, hipGetDeviceProperties(&c->prop, device));
-  if (!strstr(c->prop.gcnArchName, "gfx950")) {
-    std::string arch = c->prop.gcnArchName;
-    delete c;
-    return fail(nullptr, ZTVM_E_NODEVICE, "device %d is %s; this library holds gfx950 code only", device, arch.c_str());
-  }
+  if (!strstr(c->prop.gcnArchName, "gfx950"))
+    return fail(nullptr, ZTVM_E_NODEVICE, "device %d is %s; this library holds gfx950 code only", device, c->prop.gcnArchName);
   HIP_TRY(nullptr, hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
   c->tune.num_cus = c->prop.multiProcessorCount > 0 ? c->prop.multiProcessorCount : 256;
   {
     hipError_t e = static_scratch_of(device, &c->static_scratch);
-    if (e != hipSuccess) {
-      (void)hipStreamDestroy(c->stream);
-      delete c;
-      return fail(nullptr, ZTVM_E_HIP, "ztvm_create: address of the static scratch array: %s", hipGetErrorString(e));
-    }
+    if (e != hipSuccess) return fail(nullptr, ZTVM_E_HIP, "ztvm_create: address of the static scratch array: %s", hipGetErrorString(e));
   }
   c->scratch = std::make_shared<DevicePool>(DeviceAlloc{device});
-  if (!c->scratch->reserve(4u << 20)) {
-    (void)hipStreamDestroy(c->stream);
-    delete c;
-    return fail(nullptr, ZTVM_E_HIP, "ztvm_create: no device memory for the scratch buffer");
-  }
+  if (!c->scratch->reserve(4u << 20)) return fail(nullptr, ZTVM_E_HIP, "ztvm_create: no device memory for the scratch buffer");
+  HIP_TRY(nullptr, hipMalloc(reinterpret_cast<void**>(&c->gemm_counters), ZTVM_GEMM_SPLIT_TILES * sizeof(uint32_t)));
+  HIP_TRY(nullptr, hipMemset(c->gemm_counters, 0, ZTVM_GEMM_SPLIT_TILES * sizeof(uint32_t)));
+  g.c = nullptr;
   *out = c;
   return ZTVM_OK;
 }
@@ -358,6 +363,7 @@ void ztvm_destroy(ztvm_ctx* ctx) {
     (void)hipStreamSynchronize(ctx->stream);
     (void)hipStreamDestroy(ctx->stream);
   }
+  if (ctx->gemm_counters) (void)hipFree(ctx->gemm_counters);
   if (ctx->scratch) ctx->scratch->release_all();  // command buffers of this context are dead with it
   delete ctx;
 }
@@ -474,7 +480,9 @@ static int matmul_impl(ztvm_ctx* ctx, const ztvm_matmul_desc* desc, bool use_sta
     case ZTVM_KERNEL_ROWS:
     case ZTVM_KERNEL_SKINNY:
     case ZTVM_KERNEL_GEMM: {
-      const size_t need = fam == ZTVM_KERNEL_GEMM ? gemm_scratch_bytes(a) : (fam == ZTVM_KERNEL_ROWS ? rows_scratch_bytes(a) : skinny_scratch_bytes(a, ctx->tune));
+      // the tile GEMM's k split takes what the fixed buffer leaves after the group sums, or is not made
+      const size_t limit = use_static ? (size_t)ZTVM_STATIC_SCRATCH_BYTES : 0;
+      const size_t need = fam == ZTVM_KERNEL_GEMM ? gemm_scratch_bytes(a, ctx->tune, limit) : (fam == ZTVM_KERNEL_ROWS ? rows_scratch_bytes(a) : skinny_scratch_bytes(a, ctx->tune));
       void* scratch = nullptr;
       if (use_static) {
         if (need > (size_t)ZTVM_STATIC_SCRATCH_BYTES)
@@ -485,7 +493,7 @@ static int matmul_impl(ztvm_ctx* ctx, const ztvm_matmul_desc* desc, bool use_sta
         rc = scratch_for(ctx, need, &scratch);
         if (rc) return rc;
       }
-      if (fam == ZTVM_KERNEL_GEMM) HIP_TRY(ctx, launch_gemm(a, ctx->tune, scratch, ctx->stream));
+      if (fam == ZTVM_KERNEL_GEMM) HIP_TRY(ctx, launch_gemm(a, ctx->tune, scratch, ctx->gemm_counters, limit, ctx->stream));
       else if (fam == ZTVM_KERNEL_ROWS) HIP_TRY(ctx, launch_rows(a, ctx->tune, scratch, ctx->stream));
       else HIP_TRY(ctx, launch_skinny(a, ctx->tune, scratch, ctx->stream));
       break;
