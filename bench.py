@@ -47,15 +47,20 @@ def make_desc(capi, bits, K, N, M, bufs, kernel=0):
                            weights=bufs["w"], biases=bufs["b"])
 
 
-def upload_set(ctx, synth, K, N, bits, salt, M=1):
+def upload_set(ctx, synth, K, N, bits, salt, M=1, share_in=None):
+    """One weight set with its own output; `share_in` = (device address, host array) of an activation buffer that the
+    sets of a rotation share (the reference's bench does: one activation buffer per shape, one output per rotation
+    slot, scripts/kernel-ab-ours.mjs:97-105: in a decode loop the activations were written by the dispatch before)."""
     w = synth.packed_weights(N, K, bits=bits, salt=salt)
     s = synth.scales(N, K, salt=salt)
     b = synth.biases(N, K, s, "A", salt=salt)
-    x = synth.activations(M, K, salt=salt)
+    x = share_in[1] if share_in else synth.activations(M, K, salt=salt)
     bufs = {}
-    for key, arr in (("w", w), ("s", s), ("b", b), ("in", x)):
+    for key, arr in (("w", w), ("s", s), ("b", b)) + (() if share_in else (("in", x),)):
         bufs[key] = ctx.alloc(arr.nbytes)
         ctx.upload(bufs[key], arr)
+    if share_in:
+        bufs["in"] = share_in[0]
     bufs["out"] = ctx.alloc(M * N * 2)
     return bufs, (x, w, s, b)
 
@@ -140,6 +145,93 @@ def verify(ctx, oracle, capi, desc, host, bits, K, N, M, f16w=False):
     return err
 
 
+_MOE_STACK = {}
+
+
+def routed_ffn_five(ctx, capi, synth, tokens, salt=0):
+    """The routed FFN of configs[3] with a shared expert (257 stacked experts, 9 slots) as its five dispatches:
+    router logits (8-bit) -> softmax top-k -> gate + up + SiLU (one gated GEMV pass per pair) -> down -> combine.
+    Returns [(name, launch)]; the expert stack is uploaded once per context."""
+    E, slots, d_model, ffn = 256, 8, 2048, 512
+    E1, S = E + 1, slots + 1
+    if id(ctx) not in _MOE_STACK:
+        full_w = {}
+        for name, N_, K_ in (("gate", ffn, d_model), ("up", ffn, d_model), ("down", d_model, ffn)):
+            w = synth.packed_weights(N_, K_, experts=E1, salt=10 + len(name))
+            sc = synth.scales(N_, K_, experts=E1, salt=10 + len(name))
+            bi = synth.biases(N_, K_, sc, experts=E1, salt=10 + len(name))
+            full_w[name] = tuple(_put(ctx, a) for a in (w, sc, bi))
+        rng = np.random.default_rng(17)
+        r_w = _put(ctx, rng.integers(0, 2 ** 32, (E1, d_model // 4), dtype=np.uint64).astype(np.uint32))
+        r_sh = (rng.random((E1, d_model // 64)) * 2e-4 + 2e-4).astype(np.float16)
+        _MOE_STACK[id(ctx)] = (full_w, r_w, _put(ctx, r_sh), _put(ctx, (-127.5 * r_sh.astype(np.float32)).astype(np.float16)))
+    full_w, r_w, r_s, r_b = _MOE_STACK[id(ctx)]
+    x = _put(ctx, synth.activations(tokens, d_model, salt=600 + salt))
+    logits, ids, score = ctx.alloc(tokens * E1 * 4), ctx.alloc(tokens * S * 4), ctx.alloc(tokens * S * 4)
+    h, dn, y = ctx.alloc(tokens * S * ffn * 2), ctx.alloc(tokens * S * d_model * 2), ctx.alloc(tokens * d_model * 2)
+    common = dict(bits=4, affine=1, M=1, slots=S, tokens=tokens, ids_stride=S, experts=E1, ids=ids)
+    dgated = capi.MatmulDesc(N=ffn, k_packed=d_model // 8, scales_per_row=d_model // 64, in_slot_stride=0, in_tok_stride=d_model,
+                             in_=x, out_slot_stride=ffn, out_tok_stride=S * ffn, out=h, weights=full_w["gate"][0],
+                             scales=full_w["gate"][1], biases=full_w["gate"][2], **common)
+    dd = capi.MatmulDesc(N=d_model, k_packed=ffn // 8, scales_per_row=ffn // 64, in_slot_stride=ffn, out_slot_stride=d_model,
+                         in_tok_stride=S * ffn, out_tok_stride=S * d_model, in_=h, out=dn, weights=full_w["down"][0],
+                         scales=full_w["down"][1], biases=full_w["down"][2], **common)
+    return [("router_logits", lambda: ctx.moe_router_logits(logits, x, r_w, r_s, r_b, 8, d_model, E1, tokens)),
+            ("router_topk", lambda: ctx.moe_router_topk(ids, score, logits, E, slots, True, True, tokens)),
+            ("gate_up_silu", lambda: ctx.ffn_gated(dgated, full_w["up"][0], full_w["up"][1], full_w["up"][2])),
+            ("down", lambda: ctx.matmul(dd)),
+            ("combine", lambda: ctx.moe_combine(y, dn, score, tokens, d_model, S))]
+
+
+def f16_gemm_probe(K, N, Ms, child=False):
+    """The empirical ceiling beside the prefill GEMM: a plain f16 [M,K] x [K,N] product through the vendor library
+    (torch.matmul -> hipBLASLt) at the same shapes, rotating over three weight matrices (352 MB), six untimed and six
+    timed replays like the GEMM rows (the reference's competitor arm at the same shapes, scripts/kernel-ab-ours.mjs:
+    134-140). Measurement only: nothing of the product imports torch, and the probe runs in a process of its own
+    (torch brings its own copy of the HIP runtime). Empty if torch is not there."""
+    if not child:
+        try:
+            out = subprocess.run([sys.executable, os.path.abspath(__file__), "--f16-probe-child"], capture_output=True, text=True,
+                                 timeout=600)
+            return json.loads(out.stdout.strip().splitlines()[-1])
+        except Exception as e:   # no torch, no GPU for it, a crash of its own: the bench goes on without the rows
+            sys.stderr.write("bench: f16 probe skipped (%s)\n" % (e,))
+            return {}
+    import torch
+    rows = {}
+    ws = [torch.randn(N, K, device="cuda", dtype=torch.float16) for _ in range(3)]
+    for M in Ms:
+        a = torch.randn(M, K, device="cuda", dtype=torch.float16)
+        reps = 4 if M <= 512 else 2
+
+        def replay():
+            for _ in range(reps):
+                for w in ws:
+                    torch.matmul(a, w.t())
+
+        for _ in range(6):
+            replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        times = []
+        for _ in range(6):
+            e0.record()
+            replay()
+            e1.record()
+            torch.cuda.synchronize()
+            times.append(e0.elapsed_time(e1) / (reps * len(ws)))
+        ms = sum(times) / len(times)
+        tf = 2.0 * M * K * N / ms / 1e9
+        rows["f16_gemm_probe_M%d_K%d_N%d" % (M, K, N)] = {"us": round(ms * 1e3, 2), "TFLOP/s": round(tf, 1),
+                                                          "mfma_f16_frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
+                                                          "what": "torch.matmul f16 (vendor GEMM), weights as [N,K] f16",
+                                                          "rotation_MB": round(3 * N * K * 2 / 1e6, 1)}
+        del a
+    del ws
+    torch.cuda.empty_cache()
+    return rows
+
+
 def cpu_baseline(oracle, synth, budget_s=12.0):
     """The CPU oracle (a port of the reference's JS kernel-test reference) on this host's cores."""
     threads = oracle.max_threads()
@@ -180,13 +272,19 @@ def main():
     ap.add_argument("--sets", type=int, default=8, help="distinct weight sets rotated through (8 x 80 MB > 256 MB cache)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the per-shape, GEMM, MoE and int3 extras")
-    ap.add_argument("--pmc", nargs="?", const="base", default=None, choices=["base", "down"],
+    ap.add_argument("--no-f16-probe", action="store_true", help="skip the vendor f16 GEMM rows (they import torch)")
+    ap.add_argument("--pmc", nargs="?", const="base", default=None, choices=["base", "down", "moe"],
                     help="counter-collection mode for `rocprofv3 --pmc`: a few eager launches of a 256 MiB copy "
                          "(calibration), then (base) of each configs[1] GEMV, of the M=512 prefill GEMM and of the "
                          "small-batch families (M = 8, 32, 128), or (down) of the down projection of a 512-row "
-                         "prefill chunk (K=14336, N=4096) in the family the library picks and in the tile GEMM; no timing")
+                         "prefill chunk (K=14336, N=4096) in the family the library picks and in the tile GEMM, or (moe) of the routed "
+                         "FFN of configs[3] as five dispatches at 1 and 16 tokens and of the row-group GEMV at M=8 (int4, int3); no timing")
     ap.add_argument("--option", action="append", default=[], help="name=value launch knob (ztvm_set_option)")
+    ap.add_argument("--f16-probe-child", action="store_true", help=argparse.SUPPRESS)
     args = ap.parse_args()
+    if args.f16_probe_child:
+        print(json.dumps(f16_gemm_probe(4096, 14336, (128, 512, 2048), child=True)))
+        return
     if args.gpus != 1:
         raise SystemExit("bench.py: this path is built and measured on ONE GPU; --gpus %d is not supported "
                          "(a second GPU would own a column range of each weight matrix; nothing here uses one)" % args.gpus)
@@ -208,6 +306,21 @@ def main():
         ctx.fill(src, 1, nbytes)
         for _ in range(3):
             ctx.copy(dst, src, nbytes)
+        if args.pmc == "moe":
+            for tokens in (1, 16):
+                blocks = [routed_ffn_five(ctx, capi, synth, tokens, salt=r) for r in range(3)]
+                for r in range(6):
+                    for _, fn in blocks[r % 3]:
+                        fn()
+            K, N = 4096, 14336
+            for bits in (4, 3):
+                bdescs = [make_desc(capi, bits, K, N, 8, upload_set(ctx, synth, K, N, bits, salt=r, M=8)[0]) for r in range(2)]
+                for r in range(6):
+                    ctx.matmul(bdescs[r % 2])
+            ctx.sync()
+            ctx.close()
+            print(json.dumps({"pmc_mode": "moe", "copy_bytes": nbytes}))
+            return
         if args.pmc == "down":
             K, N, M = 14336, 4096, 512
             for kern in (capi.KERNEL_AUTO, capi.KERNEL_GEMM):
@@ -245,8 +358,10 @@ def main():
     for i, (_, K, N) in enumerate(GEMV_SHAPES):
         wb = synth.weight_bytes(N, K)
         per_set, first_host = [], None
+        x_host = synth.activations(1, K, salt=i)
+        x_shared = (_put(ctx, x_host), x_host)   # one activation vector per shape, as in a decode loop
         for r in range(max(args.sets, n_sets(wb))):
-            bufs, host = upload_set(ctx, synth, K, N, 4, salt=10 * r + i)
+            bufs, host = upload_set(ctx, synth, K, N, 4, salt=10 * r + i, share_in=x_shared)
             desc = make_desc(capi, 4, K, N, 1, bufs)
             if r == 0:
                 verify(ctx, oracle, capi, desc, host, 4, K, N, 1)
@@ -282,6 +397,7 @@ def main():
                                "per step, rotating over %.0f MB of distinct weights" % (rotation_bytes / 1e6),
                    "device": info["name"], "compute_units": info["compute_units"], "rotation_MB": round(rotation_bytes / 1e6, 1),
                    "timing": "median of %d replays of %d recorded steps, one replay in flight at a time" % (ROUNDS, args.steps),
+                   "activations": "one vector per shape shared by its weight sets, one output per set (scripts/kernel-ab-ours.mjs:97-105)",
                    "ms_per_step_min": round(rounds[0] / args.steps, 6), "ms_per_step_max": round(rounds[-1] / args.steps, 6),
                    "clocks": clocks()},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -356,8 +472,19 @@ def main():
             ms = timed_graph(ctx, [lambda d=descs[j % ng]: ctx.matmul(d) for j in range(reps * ng)], reps=6, warm=6) / (reps * ng)
             tf = 2.0 * M * 4096 * 14336 / ms / 1e9
             extra["gemm_M%d_K4096_N14336" % M] = {"us": round(ms * 1e3, 2), "TFLOP/s": round(tf, 1),
-                                                  "mfma_f16_frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
+                                                  "mfma_f16_frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4), "family": "gemm (forced)",
                                                   "rotation_MB": round(ng * (g_wb + M * 4096 * 2) / 1e6, 1)}
+            # the same dispatch with the family left to the library
+            adescs = [make_desc(capi, 4, 4096, 14336, M, b) for b, _ in gsets]
+            fam = capi.KERNEL_NAMES[capi.resolve(adescs[0])]
+            if fam != "gemm":
+                verify(ctx, oracle, capi, adescs[0], gsets[0][1], 4, 4096, 14336, M)
+                ms = timed_graph(ctx, [lambda d=adescs[j % ng]: ctx.matmul(d) for j in range(reps * ng)], reps=6, warm=6) / (reps * ng)
+                tf = 2.0 * M * 4096 * 14336 / ms / 1e9
+            extra["gemm_M%d_K4096_N14336_auto" % M] = {"us": round(ms * 1e3, 2), "TFLOP/s": round(tf, 1),
+                                                       "mfma_f16_frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4), "family": fam}
+        if not args.no_f16_probe:
+            extra.update(f16_gemm_probe(4096, 14336, (128, 512, 2048)))
         # the down projection of the same prefill chunk (K=14336 -> N=4096, M=512): 32 column tiles, where the family
         # choice goes by an estimate of both kernels; the library's choice beside the tile GEMM forced. Weights: the
         # headline's rotating sets of this shape; one activation buffer, one output per set
@@ -527,7 +654,8 @@ def main():
             x = _put(ctx, synth.activations(tokens, d_model, salt=5))
             gu = ctx.alloc(tokens * slots * 2 * ffn * 2)
             out = ctx.alloc(tokens * slots * d_model * 2)
-            trios = []
+            hf, out_f = ctx.alloc(tokens * slots * ffn * 2), ctx.alloc(tokens * slots * d_model * 2)
+            trios, pairs = [], []
             for ids in id_sets:
                 d_ids = _put(ctx, ids)
                 gcommon = dict(bits=4, affine=1, M=1, N=ffn, k_packed=d_model // 8, scales_per_row=d_model // 64, slots=slots,
@@ -540,14 +668,42 @@ def main():
                                      out_tok_stride=slots * d_model, ids_stride=slots, experts=E, out=out, in_=gu, ids=d_ids,
                                      weights=moe_w["down"][0], scales=moe_w["down"][1], biases=moe_w["down"][2])
                 trios.append((dg, du, dd))
+                # the same block as two launches: gate + up + SiLU in one pass over the token's activations, then down
+                fcommon = dict(gcommon, out_slot_stride=ffn, out_tok_stride=slots * ffn)
+                dgu = capi.MatmulDesc(out=hf, weights=moe_w["gate"][0], scales=moe_w["gate"][1], biases=moe_w["gate"][2], **fcommon)
+                ddf = capi.MatmulDesc(bits=4, affine=1, M=1, N=d_model, k_packed=ffn // 8, scales_per_row=ffn // 64, slots=slots,
+                                      tokens=tokens, in_slot_stride=ffn, out_slot_stride=d_model, in_tok_stride=slots * ffn,
+                                      out_tok_stride=slots * d_model, ids_stride=slots, experts=E, out=out_f, in_=hf, ids=d_ids,
+                                      weights=moe_w["down"][0], scales=moe_w["down"][1], biases=moe_w["down"][2])
+                pairs.append((dgu, ddf))
             nrep = 2 * len(trios)
             ms = timed_graph(ctx, [lambda d=d_: ctx.matmul(d) for r in range(nrep) for d_ in trios[r % len(trios)]], reps=3) / nrep
             per_replay = [len(set(int(v) for v in ids.reshape(-1))) for ids in id_sets]
             union = len(set(int(v) for ids in id_sets for v in ids.reshape(-1)))
             distinct = float(np.mean(per_replay))
-            extra["moe_block_tokens%d" % tokens] = {"us": round(ms * 1e3, 2), "pairs": tokens * slots, "distinct_experts": round(distinct, 1),
+            extra["moe_block_tokens%d" % tokens] = {"us": round(ms * 1e3, 2), "launches": 3, "pairs": tokens * slots, "distinct_experts": round(distinct, 1),
                                                      "expert_GB/s": round(distinct * per_expert / ms / 1e6, 1),
+                                                     "hbm_frac": round(distinct * per_expert / ms / 1e6 / HBM_PEAK_GBS, 4),
                                                      "rotation_MB": round(union * per_expert / 1e6, 1)}
+
+            def fused_block(pr):
+                ctx.ffn_gated(pr[0], moe_w["up"][0], moe_w["up"][1], moe_w["up"][2])
+                ctx.matmul(pr[1])
+
+            # checked against the three-launch form before it is timed: down(silu(gate) * up) of the same experts
+            for d_ in trios[0]:
+                ctx.matmul(d_)
+            fused_block(pairs[0])
+            g_u = ctx.download(gu, tokens * slots * 2 * ffn * 2, np.float16).astype(np.float32).reshape(tokens * slots, 2, ffn)
+            h_ref = (g_u[:, 1] * (g_u[:, 0] / (1.0 + np.exp(-g_u[:, 0])))).astype(np.float64)
+            h_got = ctx.download(hf, tokens * slots * ffn * 2, np.float16).astype(np.float64).reshape(tokens * slots, ffn)
+            if not np.all(np.isfinite(h_got)) or float(np.max(np.abs(h_got - h_ref) / (np.abs(h_ref) + 1e-2))) > 1e-2:
+                raise SystemExit("bench: two-launch MoE block disagrees with the three-launch form (tokens=%d)" % tokens)
+            ms = timed_graph(ctx, [lambda pr=pairs[r % len(pairs)]: fused_block(pr) for r in range(nrep)], reps=3) / nrep
+            extra["moe_block_fused_tokens%d" % tokens] = {"us": round(ms * 1e3, 2), "launches": 2, "pairs": tokens * slots,
+                                                           "expert_GB/s": round(distinct * per_expert / ms / 1e6, 1),
+                                                           "hbm_frac": round(distinct * per_expert / ms / 1e6 / HBM_PEAK_GBS, 4),
+                                                           "rotation_MB": round(union * per_expert / 1e6, 1)}
         # the whole routed FFN of configs[3] with a shared expert (257 stacked experts, 9 slots): router logits
         # (8-bit) -> softmax top-k -> gate, up -> silu_mul -> down -> combine, routed on the device
         E1, S = E + 1, slots + 1

@@ -180,6 +180,21 @@ def test_many_row_tiles(ctx, capi, synth, oracle, M, N, K, affine, bits):
     assert rel_err(y, gemm[rows].view(np.float16).astype(np.float64), 1e-2) < (6e-3 if bits == 8 else 2e-3)
 
 
+def test_default_split_follows_the_row_count(ctx, capi, synth, oracle):
+    """With the default knobs the transfer-engine kernel deals k to as many workgroups as fill one round of the CUs,
+    and the number of row tiles enters that count: at K=4096, N=4096 a row travels with 40 rows in eight k parts and
+    with 100 rows in four. Same row, another f32 summation order: the last f16 bit or two, held to a stated
+    tolerance here (pin `skinny.ksplit` for bit-stable rows across M; test_ragged_skinny does)."""
+    M, CAP, N, K = 40, 100, 4096, 4096
+    A, w, s, b = make(synth, 4, True, CAP, N, K)
+    small = run(ctx, capi, 4, True, M, M, N, K, A[:M], w, s, b, capi.KERNEL_SKINNY).view(np.float16).astype(np.float64)
+    big = run(ctx, capi, 4, True, CAP, CAP, N, K, A, w, s, b, capi.KERNEL_SKINNY).view(np.float16).astype(np.float64)
+    assert rel_err(small, big[:M], 1e-2) < 2e-3
+    rows = np.array([0, 17, M - 1])
+    ref = oracle.gemm(oracle.MODE_FORMULA_F64, 4, True, len(rows), N, K, np.ascontiguousarray(A[rows]), w, s, b, threads=8)
+    assert rel_err(small[rows], ref, 1e-2) < 1e-2 and rel_err(big[rows], ref, 1e-2) < 1e-2
+
+
 def test_auto_picks_skinny(capi):
     for M, want in ((1, capi.KERNEL_GEMV), (17, capi.KERNEL_SKINNY), (128, capi.KERNEL_SKINNY)):
         desc = capi.MatmulDesc(bits=4, affine=1, M=M, N=256, k_packed=64, scales_per_row=8, out=4096, in_=4096, scales=4096,

@@ -61,3 +61,27 @@ def test_static_scratch_refuses_what_does_not_fit(ctx, capi, synth):
             ctx.set_option("skinny.ksplit", 0)
         assert e.value.code == capi.E_UNSUPPORTED and "static buffer holds" in str(e.value)
         assert (ctx.download(out, M * N * 2, np.uint8) == 0x5A).all()
+
+
+def test_static_entry_leaves_the_scratch_pool_alone(capi, synth):
+    """What the entry point is for: on a fresh context (4 MiB pool) a dispatch that needs 8 MiB of scratch runs through
+    ztvm_matmul_static, and afterwards the pool is still 4 MiB: the same dispatch through ztvm_matmul inside a
+    recording (which cannot allocate) is refused with the pool's size in the message."""
+    M, N, K = 512, 1024, 4096   # tile GEMM with its k split: 16 tiles x 4 parts x 128 KiB of f32 totals
+    with capi.Context(0) as fresh:
+        with Dev(fresh) as d:
+            out = d.empty(M * N * 2, fill=0)
+            s = synth.scales(N, K)
+            desc = capi.MatmulDesc(bits=4, affine=1, kernel=capi.KERNEL_GEMM, M=M, N=N, k_packed=K // 8, scales_per_row=K // 64,
+                                   out=out, in_=d.put(synth.activations(M, K)), scales=d.put(s), weights=d.put(synth.packed_weights(N, K)),
+                                   biases=d.put(synth.biases(N, K, s)))
+            fresh.matmul_static(desc)
+            fresh.sync()
+            assert fresh.download(out, M * N * 2, np.uint16).any()
+            fresh.record_begin()
+            try:
+                with pytest.raises(capi.ZtvmError) as e:
+                    fresh.matmul(desc)
+            finally:
+                fresh.cmdbuf_destroy(fresh.record_end())
+            assert e.value.code == capi.E_UNSUPPORTED and "have 4194304" in str(e.value), str(e.value)

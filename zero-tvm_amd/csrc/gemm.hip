@@ -169,11 +169,11 @@ constexpr int SCB = 6;  // steps per batch of scales: two turns of the three LDS
 // else in these kernels uses M0.
 __device__ __forceinline__ void dma16(const void* base_uniform, uint32_t off, uint32_t lds_uniform) {
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base_uniform), "s"(lds_uniform)
-               : "memory");
+               : "memory", "m0");
 }
 // The same with 4 bytes per lane: LDS slot lds + 4 * lane.
 __device__ __forceinline__ void dma4(const void* base_uniform, uint32_t off, uint32_t lds_uniform) {
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(off), "s"(base_uniform), "s"(lds_uniform) : "memory");
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(off), "s"(base_uniform), "s"(lds_uniform) : "memory", "m0");
 }
 
 // Work that shares a step with the 16 matrix instructions, by half-slot hs = 2 * pair + (0 after

@@ -37,10 +37,10 @@ namespace {
 // stage is refilled only after the barrier that follows its last read, and read only after the wait and the barrier
 // that follow its transfers) is kept by the wait and barrier statements, which are.
 __device__ __forceinline__ void xfer16(const void* base, uint32_t voff, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(base), "s"(lds_base));
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(base), "s"(lds_base) : "m0");
 }
 __device__ __forceinline__ void xfer4(const void* base, uint32_t voff, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" : : "v"(voff), "s"(base), "s"(lds_base));
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" : : "v"(voff), "s"(base), "s"(lds_base) : "m0");
 }
 
 // weight rows of 64 bytes: a 128-bit read serves 8 lanes a cycle, rows of equal parity share a bank half
