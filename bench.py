@@ -461,8 +461,10 @@ def main():
         # prefill GEMM (configs[2]): K=4096, N=14336, M in {128, 512, 2048}
         gsets = []
         g_wb = synth.weight_bytes(14336, 4096)
+        gx_host = synth.activations(2048, 4096, salt=100)
+        gx = (_put(ctx, gx_host), gx_host)   # one activation buffer for every weight set of the rotation
         for r in range(n_sets(g_wb)):
-            bufs, host = upload_set(ctx, synth, 4096, 14336, 4, salt=100 + r, M=2048)
+            bufs, host = upload_set(ctx, synth, 4096, 14336, 4, salt=100 + r, M=2048, share_in=gx)
             gsets.append((bufs, host))
         ng = len(gsets)
         for M in (128, 512, 2048):
@@ -473,7 +475,7 @@ def main():
             tf = 2.0 * M * 4096 * 14336 / ms / 1e9
             extra["gemm_M%d_K4096_N14336" % M] = {"us": round(ms * 1e3, 2), "TFLOP/s": round(tf, 1),
                                                   "mfma_f16_frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4), "family": "gemm (forced)",
-                                                  "rotation_MB": round(ng * (g_wb + M * 4096 * 2) / 1e6, 1)}
+                                                  "rotation_MB": round((ng * g_wb + M * 4096 * 2) / 1e6, 1)}
             # the same dispatch with the family left to the library
             adescs = [make_desc(capi, 4, 4096, 14336, M, b) for b, _ in gsets]
             fam = capi.KERNEL_NAMES[capi.resolve(adescs[0])]
@@ -508,7 +510,9 @@ def main():
         # int3 decode GEMV (configs[4], M=1)
         wb = synth.weight_bytes(14336, 4096, bits=3)
         n3 = n_sets(wb)
-        i3 = [upload_set(ctx, synth, 4096, 14336, 3, salt=200 + r) for r in range(n3)]
+        x3_host = synth.activations(1, 4096, salt=200)
+        x3 = (_put(ctx, x3_host), x3_host)
+        i3 = [upload_set(ctx, synth, 4096, 14336, 3, salt=200 + r, share_in=x3) for r in range(n3)]
         d3 = [make_desc(capi, 3, 4096, 14336, 1, b) for b, _ in i3]
         verify(ctx, oracle, capi, d3[0], i3[0][1], 3, 4096, 14336, 1)
         ms = timed_graph(ctx, [lambda d=d3[j % n3]: ctx.matmul(d) for j in range(16 * n3)], reps=ROUNDS, rounds=True)[ROUNDS // 2] / (16 * n3)
@@ -619,7 +623,9 @@ def main():
                 host0 = gsets[0][1]
             else:
                 if (bits, "sets") not in other_sets:   # one rotation per width, built for the largest M it is used at
-                    other_sets[(bits, "sets")] = [upload_set(ctx, synth, 4096, 14336, bits, salt=300 + 10 * bits + r, M=512)
+                    ox_host = synth.activations(512, 4096, salt=300 + bits)
+                    ox = (_put(ctx, ox_host), ox_host)
+                    other_sets[(bits, "sets")] = [upload_set(ctx, synth, 4096, 14336, bits, salt=300 + 10 * bits + r, M=512, share_in=ox)
                                                   for r in range(n_sets(wb))]
                 other = other_sets[(bits, "sets")]
                 descs = [make_desc(capi, bits, 4096, 14336, M, b) for b, _ in other]

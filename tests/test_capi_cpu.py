@@ -188,3 +188,20 @@ def test_no_device_is_a_loud_error(capi):
     env = dict(os.environ, HIP_VISIBLE_DEVICES="-1", ROCR_VISIBLE_DEVICES="-1")
     out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=env, timeout=120).stdout
     assert "ERR -4" in out, out
+
+
+def test_failed_create_hands_out_nothing(capi):
+    """Every failing exit of ztvm_create leaves *out null (so a caller that ignores the code cannot use or leak a
+    half-built context) and says why; a null out pointer is refused."""
+    import subprocess, sys
+    code = ("import ctypes as C, importlib, sys; sys.path.insert(0,%r)\n"
+            "c = importlib.import_module('zero-tvm_amd.host.capi'); L = c.load()\n"
+            "for i in range(50):\n"
+            "  h = C.c_void_p(0xDEAD)\n"
+            "  rc = L.ztvm_create(0, C.byref(h)); assert rc == -4 and not h.value, (rc, h.value)\n"
+            "  assert b'no HIP device' in L.ztvm_last_error(None)\n"
+            "assert L.ztvm_create(0, None) == -1\n"
+            "L.ztvm_destroy(None); print('FINE')") % ROOT
+    env = dict(os.environ, HIP_VISIBLE_DEVICES="-1", ROCR_VISIBLE_DEVICES="-1")
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=env, timeout=120)
+    assert "FINE" in r.stdout, r.stdout + r.stderr

@@ -176,14 +176,16 @@ def test_config3_shape(ctx, capi, synth, oracle, M):
     K, N = 4096, 14336
     A, w, s, b = make(synth, True, M, N, K)
     got = run(ctx, capi, True, M, M, N, K, A, w, s, b, capi.KERNEL_GEMM)
-    rows = np.array([0, 1, M // 2, M - 1])   # first and last tile row of the grid (M=2048: 8 tile rows, 3.5 rounds of workgroups)
+    # one row of every 256-row tile (at a different place in each), and the first and last row of the matrix: M=2048 is
+    # 8 tile rows in 3.5 rounds of workgroups, the last half round split along k
+    rows = np.unique(np.concatenate([[0, 1, M - 1], [min(t + (37 * (t // 256 + 1)) % 256, M - 1) for t in range(0, M, 256)]]))
     y = got[rows].view(np.float16).astype(np.float64)
     ref = oracle.gemm(oracle.MODE_FORMULA_F64, 4, True, len(rows), N, K, A[rows], w, s, b, threads=8)
     e = rel_err(y, ref, 1e-2)
     print("M=%d: rel err vs formula %.2e" % (M, e))
     assert e < 1e-2
     # every row agrees with the GEMV family's answer for the same row (two independent kernels)
-    gv = run(ctx, capi, True, 4, 4, N, K, A[rows], w, s, b, capi.KERNEL_GEMV)
+    gv = run(ctx, capi, True, len(rows), len(rows), N, K, A[rows], w, s, b, capi.KERNEL_GEMV)
     assert rel_err(y, gv.view(np.float16).astype(np.float64), 1e-2) < 1e-2
 
 

@@ -272,6 +272,10 @@ bool gemv_stream_supports(const MatmulArgs& a, const Tune& t) {
   if (a.slots != 0 || a.up_weights || a.qkv || a.delta) return false;
   if (!(a.bits == 4 || (a.bits == 3 && a.affine))) return false;
   if (a.K == 0 || a.K % 32u) return false;
+  // buffer resources carry 32-bit byte counts, and the out-of-range offset that stands for "no row" (2 GiB) must lie
+  // past every array for its loads to return zeros
+  const uint64_t lim = 1ull << 31;
+  if ((uint64_t)a.N * a.k_packed * 4 >= lim || (uint64_t)a.N * a.spr * 2 >= lim) return false;
   const uint32_t passes = passes_of(a);
   if (passes > 16) return false;
   const uint32_t kparts = kparts_of(passes);
