@@ -10,7 +10,8 @@ streams its weights from HBM. Inputs are resident in HBM before timing.
 Timing discipline (the reference's, scripts/kernel-ab-ours.mjs:75-99): outputs are validated against the
 oracle before anything is timed; every memory-bound row rotates over more than 256 MB of distinct
 operands (`rotation_MB` in the row); the headline is the median of ROUNDS timed replays of the recorded
-steps, one replay in flight at a time, with min and max beside it; a plain streaming read of the same
+steps (HIP events around each, each queued behind an untimed replay so that the host's
+hand-over of the command buffer is not in the timed region), with min and max beside it; a plain streaming read of the same
 byte count is timed the same way in the same run (`extra.hbm_read_probe_*`); clocks are recorded.
 
 Prints ONE JSON line: value = algorithmic weight GB/s over the timed steps,
@@ -74,23 +75,28 @@ def _put(ctx, arr):
 def timed_graph(ctx, launches, reps=1, warm=1, rounds=False):
     """Record `launches` (callables) into one command buffer, replay `warm` times untimed, then time `reps` replays.
     Returns the mean milliseconds per replay, or with rounds=True the sorted list of the replays' times.
+    Every timed replay is queued right behind an untimed replay of the same command buffer, with the two events
+    around the second: the host needs some 25 us to hand a recorded command buffer to the GPU, and with nothing
+    queued ahead the GPU would sit idle for that long inside the timed region (6 % of a replay of 20 steps; the
+    kernels are what is measured, as the time stamps of a kernel trace measure them). The replays of a pair run one
+    after the other on the stream, and the pair is waited for before the next is submitted.
     Compute-bound rows pass warm > 1: after an idle stretch (the oracle check before a row is one) the clock takes
     tens of milliseconds of load to come back up (the M=512 GEMM: 88 us cold, 76 after a few ms, 72 sustained)."""
     ctx.record_begin()
     for fn in launches:
         fn()
     cb = ctx.record_end()
-    # one replay in flight at a time: each is waited for before the next is submitted
     for _ in range(warm):
         ctx.submit(cb)
         ctx.sync()
     e0, e1 = ctx.event(), ctx.event()
     times = []
     for _ in range(reps):
+        ctx.submit(cb)                          # untimed: keeps the GPU busy while the host queues what follows
         ctx.event_record(e0)
         ctx.submit(cb)
         ctx.event_record(e1)
-        times.append(ctx.elapsed_ms(e0, e1))   # waits for the replay: one in flight at a time
+        times.append(ctx.elapsed_ms(e0, e1))   # waits for the pair
     ctx.event_destroy(e0)
     ctx.event_destroy(e1)
     ctx.cmdbuf_destroy(cb)
@@ -396,7 +402,7 @@ def main():
         "config": {"workload": "configs[1]: int4 affine g64 decode GEMV, M=1, (4096->14336)+(14336->4096)+(4096->6144) "
                                "per step, rotating over %.0f MB of distinct weights" % (rotation_bytes / 1e6),
                    "device": info["name"], "compute_units": info["compute_units"], "rotation_MB": round(rotation_bytes / 1e6, 1),
-                   "timing": "median of %d replays of %d recorded steps, one replay in flight at a time" % (ROUNDS, args.steps),
+                   "timing": "median of %d replays of %d recorded steps, HIP events around each, each queued behind an untimed replay" % (ROUNDS, args.steps),
                    "activations": "one vector per shape shared by its weight sets, one output per set (scripts/kernel-ab-ours.mjs:97-105)",
                    "ms_per_step_min": round(rounds[0] / args.steps, 6), "ms_per_step_max": round(rounds[-1] / args.steps, 6),
                    "clocks": clocks()},

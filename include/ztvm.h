@@ -189,7 +189,8 @@ ZTVM_API int ztvm_matmul(ztvm_ctx* ctx, const ztvm_matmul_desc* desc);
  * ZTVM_E_UNSUPPORTED and a message that says how much (ztvm_matmul takes any size); where AUTO would
  * give a dispatch of more than 128 rows to the skinny family and its reordered copy of the
  * activations (M x K f16) outgrows the array, the tile GEMM runs it instead (results then agree
- * with ztvm_matmul's to the last f16 bit or two, not bit for bit). Nothing in the
+ * with ztvm_matmul's to the last f16 bit or two, not bit for bit); likewise the tile GEMM runs
+ * without its split along k where the f32 totals the parts exchange would outgrow the array. Nothing in the
  * array has to start at zero: every kernel writes what it later reads. All calls on one GPU share
  * the array, from every context and thread: two ztvm_matmul_static dispatches that overlap on one
  * GPU (different contexts or streams) race on it; dispatches on one context are ordered and safe. */
@@ -366,7 +367,12 @@ ZTVM_API int ztvm_event_elapsed_ms(ztvm_ctx* ctx, ztvm_event* start, ztvm_event*
 /* ---- launch tuning -------------------------------------------------------- */
 
 /* Named integer knobs for measurement sweeps (e.g. "gemv.wg_per_cu"). Unknown
- * names are ZTVM_E_INVALID. Defaults are the measured best. */
+ * names are ZTVM_E_INVALID. Defaults are the measured best. Three of them decide the f32 summation
+ * order over k and so the last f16 bit or two of a result: "skinny.ksplit" and "skinny.shape" (0 =
+ * chosen from M, N and K: the same row may then be summed differently in dispatches of different M)
+ * and "gemm.split" (0 = the tile GEMM deals the tiles of a last round of workgroups that fills at
+ * most half the CUs to several workgroups along k, which add their f32 totals in a fixed order; 1 =
+ * never). Pin them for rows that must not depend on the batch they travel in. */
 ZTVM_API int ztvm_set_option(ztvm_ctx* ctx, const char* name, int value);
 ZTVM_API int ztvm_get_option(ztvm_ctx* ctx, const char* name, int* value);
 
