@@ -351,6 +351,7 @@ int ztvm_create(int device, ztvm_ctx** out) {
   if (!c->scratch->reserve(4u << 20)) return fail(nullptr, ZTVM_E_HIP, "ztvm_create: no device memory for the scratch buffer");
   HIP_TRY(nullptr, hipMalloc(reinterpret_cast<void**>(&c->gemm_counters), ZTVM_GEMM_SPLIT_TILES * sizeof(uint32_t)));
   HIP_TRY(nullptr, hipMemset(c->gemm_counters, 0, ZTVM_GEMM_SPLIT_TILES * sizeof(uint32_t)));
+  HIP_TRY(nullptr, hipDeviceSynchronize());  // the fill runs on the null stream, which the context's stream does not wait for
   g.c = nullptr;
   *out = c;
   return ZTVM_OK;
