@@ -241,7 +241,6 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
   // the parts' f32 totals in part order, so a tile's result does not depend on who arrives when.
   // (the split tiles run as a launch of their own, SPLIT, after the whole ones)
   uint32_t id = blockIdx.x, kpart = 0;
-  constexpr bool split = SPLIT;
   if (SPLIT) {
     id = p.full_tiles + blockIdx.x / p.parts;
     kpart = blockIdx.x % p.parts;
